@@ -9,6 +9,8 @@
 //                  (gemma4_layer_exec.rs:801-804, paged_attention_sm89.cu:96-105)
 //   score          s = scale * sum_d q[d] * k[j,d]          (paged_attention_sm89.cu:125-137)
 //   grouping       kv_head = head / (nq / nkv)              (paged_attention_sm89.cu:71)
+//   sink           with `sinks`, head h's sum of exponentials has one more term e^(sinks[h]): no key, no value,
+//                  not scaled, counted once
 //   softmax * V    m' = max(m, s); acc = acc*e^(m-m') + e^(s-m')*v; l likewise; out = acc / l
 //                  (paged_attention_sm89.cu:145-157)
 // Scores, softmax and the weighted sum are 32-bit.  Tiles start at the first
@@ -30,7 +32,8 @@ __global__ void paged_attention_generic_kernel(const T* __restrict__ q, const T*
                                                const T* __restrict__ v_pages, const int* __restrict__ block_table,
                                                int table_width, const int* __restrict__ positions,
                                                const int* __restrict__ token_req, T* __restrict__ out, int nq, int nkv,
-                                               int hd, int page_size, int num_pages, int window, float scale) {
+                                               int hd, int page_size, int num_pages, int window, float scale,
+                                               const float* __restrict__ sinks) {
   __shared__ float q_s[ATT_MAX_HD];
   __shared__ float p_s[RV_WAVE];
   __shared__ int page_s[RV_WAVE];
@@ -97,6 +100,8 @@ __global__ void paged_attention_generic_kernel(const T* __restrict__ q, const T*
     }
   }
   T* o = out + ((size_t)t * nq + h) * hd;
+  // a sink: one more term e^(sink - m) in the sum of the head's exponentials, with no key and no value
+  if (sinks != nullptr) l += expf(sinks[h] - m);
   const float inv_l = 1.0f / l;
 #pragma unroll
   for (int i = 0; i < ATT_DIMS_PER_LANE; ++i) {
@@ -108,7 +113,8 @@ __global__ void paged_attention_generic_kernel(const T* __restrict__ q, const T*
 extern "C" int rv_paged_attention_generic(hipStream_t stream, const void* q, const void* k_pages, const void* v_pages,
                                           const int* block_table, int table_width, const int* positions,
                                           const int* token_req, void* out, int dtype, int num_tokens, int nq, int nkv,
-                                          int hd, int page_size, int num_pages, int window, float scale) {
+                                          int hd, int page_size, int num_pages, int window, float scale,
+                                          const float* sinks) {
   RV_CHECK(num_tokens >= 0 && nq > 0 && nkv > 0 && nq % nkv == 0, "attention: bad head counts nq=%d nkv=%d", nq, nkv);
   RV_CHECK(hd > 0 && hd <= ATT_MAX_HD, "attention: head_dim %d must be in 1..%d", hd, ATT_MAX_HD);
   RV_CHECK(page_size > 0 && num_pages > 0 && table_width > 0, "attention: bad cache geometry");
@@ -120,11 +126,11 @@ extern "C" int rv_paged_attention_generic(hipStream_t stream, const void* q, con
   if (dtype == RV_F32)
     paged_attention_generic_kernel<float><<<grid, block, 0, stream>>>(
         (const float*)q, (const float*)k_pages, (const float*)v_pages, block_table, table_width, positions, token_req,
-        (float*)out, nq, nkv, hd, page_size, num_pages, window, scale);
+        (float*)out, nq, nkv, hd, page_size, num_pages, window, scale, sinks);
   else if (dtype == RV_BF16)
     paged_attention_generic_kernel<bf16_t><<<grid, block, 0, stream>>>(
         (const bf16_t*)q, (const bf16_t*)k_pages, (const bf16_t*)v_pages, block_table, table_width, positions,
-        token_req, (bf16_t*)out, nq, nkv, hd, page_size, num_pages, window, scale);
+        token_req, (bf16_t*)out, nq, nkv, hd, page_size, num_pages, window, scale, sinks);
   else
     return rv_fail("attention: unsupported dtype %d", dtype);
   RV_LAUNCH_CHECK("paged_attention_generic");

@@ -66,6 +66,46 @@ extern "C" int rv_embed_gather(hipStream_t stream, const void* table, int table_
 }
 
 // ---------------------------------------------------------------------------
+// embedding with a learned position vector: out[t,:] = table[ids[t],:] * scale + pos[positions[t],:], the sum in
+// 32-bit.  A position outside the table adds nothing (the host holds requests to the table's length).
+// ---------------------------------------------------------------------------
+template <typename TT, typename TO>
+__global__ void embed_positions_kernel(const TT* __restrict__ table, const TT* __restrict__ pos_table,
+                                       const int* __restrict__ ids, const int* __restrict__ positions,
+                                       TO* __restrict__ out, int hidden, int vocab, int max_pos, float scale) {
+  const int t = blockIdx.x;
+  const int id = ids[t];
+  const int p = positions[t];
+  TO* o = out + (size_t)t * hidden;
+  const bool id_ok = id >= 0 && id < vocab, p_ok = p >= 0 && p < max_pos;
+  const TT* row = table + (size_t)(id_ok ? id : 0) * hidden;
+  const TT* prow = pos_table + (size_t)(p_ok ? p : 0) * hidden;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+    const float e = id_ok ? rv_to_float(row[i]) * scale : 0.f;
+    o[i] = rv_from_float<TO>(p_ok ? e + rv_to_float(prow[i]) : e);
+  }
+}
+
+extern "C" int rv_embed_positions(hipStream_t stream, const void* table, const void* pos_table, int table_dtype,
+                                  const int* ids, const int* positions, void* out, int out_dtype, int num_tokens,
+                                  int hidden, int vocab, int max_pos, float scale) {
+  RV_CHECK(num_tokens >= 0 && hidden > 0 && vocab > 0 && max_pos > 0, "embed_positions: bad sizes T=%d H=%d V=%d P=%d",
+           num_tokens, hidden, vocab, max_pos);
+  if (num_tokens == 0) return 0;
+  dim3 grid(num_tokens), block(256);
+#define RV_EP(TT, TO)                                                                                              \
+  embed_positions_kernel<TT, TO><<<grid, block, 0, stream>>>((const TT*)table, (const TT*)pos_table, ids, positions, \
+                                                             (TO*)out, hidden, vocab, max_pos, scale)
+  if (table_dtype == RV_F32 && out_dtype == RV_F32) RV_EP(float, float);
+  else if (table_dtype == RV_BF16 && out_dtype == RV_BF16) RV_EP(bf16_t, bf16_t);
+  else if (table_dtype == RV_BF16 && out_dtype == RV_F32) RV_EP(bf16_t, float);
+  else return rv_fail("embed_positions: unsupported dtypes %d -> %d", table_dtype, out_dtype);
+#undef RV_EP
+  RV_LAUNCH_CHECK("embed_positions");
+  return 0;
+}
+
+// ---------------------------------------------------------------------------
 // Row kernels keep a row in registers: one block per row, a thread owns E
 // groups of V consecutive elements (V = 16 bytes' worth when the width allows,
 // else 1), so a row is read once and written once whatever the number of
@@ -499,6 +539,39 @@ extern "C" int rv_gated_act(hipStream_t stream, const void* gu, int slices, long
 #undef RV_GA_A
 #undef RV_GA
   RV_LAUNCH_CHECK("gated_act");
+  return 0;
+}
+
+// ---------------------------------------------------------------------------
+// clamped gated activation: g = min(gate, limit), u = clamp(up, -limit, limit), out = g * sigmoid(alpha * g) * (u + 1)
+// gates and ups lie in halves of a row of gu [rows, 2 * inter] (gate i at i, up i at inter + i).
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ void clamped_glu_kernel(const T* __restrict__ gu, T* __restrict__ out, int inter, long long total,
+                                   float limit, float alpha) {
+  const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= total) return;
+  const long long t = idx / inter;
+  const int i = (int)(idx - t * inter);
+  const float gate = fminf(rv_to_float(gu[(size_t)t * 2 * inter + i]), limit);
+  const float up = fminf(fmaxf(rv_to_float(gu[(size_t)t * 2 * inter + inter + i]), -limit), limit);
+  out[idx] = rv_from_float<T>(gate / (1.0f + expf(-alpha * gate)) * (up + 1.0f));
+}
+
+extern "C" int rv_clamped_glu(hipStream_t stream, const void* gu, void* out, int dtype, int rows, int inter,
+                              float limit, float alpha) {
+  RV_CHECK(rows >= 0 && inter > 0 && limit > 0.f, "clamped_glu: bad arguments rows=%d inter=%d limit=%g", rows, inter,
+           (double)limit);
+  if (rows == 0) return 0;
+  const long long total = (long long)rows * inter;
+  dim3 grid(rv_div_up(total, 256)), block(256);
+  if (dtype == RV_F32)
+    clamped_glu_kernel<float><<<grid, block, 0, stream>>>((const float*)gu, (float*)out, inter, total, limit, alpha);
+  else if (dtype == RV_BF16)
+    clamped_glu_kernel<bf16_t><<<grid, block, 0, stream>>>((const bf16_t*)gu, (bf16_t*)out, inter, total, limit, alpha);
+  else
+    return rv_fail("clamped_glu: unsupported dtype %d", dtype);
+  RV_LAUNCH_CHECK("clamped_glu");
   return 0;
 }
 

@@ -1,0 +1,108 @@
+// Routing for a mixture of experts whose experts are chosen by the token's id: a table [vocab, top] names each
+// id's experts.  Nothing here waits for the host: the sorted order is made on the device, with room for the worst
+// case, so a step's launches do not depend on the tokens and can be replayed from a graph.
+//
+//   moe_route     sorts the step's (token, choice) pairs by expert.  Each expert's rows start at a multiple of
+//                 `tile` rows (the grouped product takes a tile of rows against one expert's matrix):
+//                   slot_of[t * top + k]   the sorted row of token t's k-th choice
+//                   row_token[r]           the token of sorted row r, -1 for the filling rows
+//                   tile_group[r / tile]   the expert of a tile of rows, -1 for tiles past the last expert's
+//                 `capacity` rows (a multiple of tile) hold every case: tokens * top + experts * (tile - 1) at most.
+//   moe_combine   out[t] = weight * sum_k y[slot_of[t * top + k]] (+ shared[t]), the sum in 32-bit, choices in order
+//
+// The place of a row inside its expert's rows depends on the order in which the threads arrive; each row's result
+// does not, since the products work row by row.
+#include "common.h"
+
+#define MOE_MAX_EXPERTS 1024
+#define MOE_THREADS 1024
+
+__global__ void __launch_bounds__(MOE_THREADS)
+moe_route_kernel(const int* __restrict__ token_ids, int num_tokens, const int* __restrict__ table, int vocab, int top,
+                 int experts, int tile, int capacity, int* __restrict__ slot_of, int* __restrict__ row_token,
+                 int* __restrict__ tile_group) {
+  __shared__ int count[MOE_MAX_EXPERTS];
+  __shared__ int first[MOE_MAX_EXPERTS];
+  const int tid = threadIdx.x;
+  const int slots = num_tokens * top;
+  for (int e = tid; e < experts; e += MOE_THREADS) count[e] = 0;
+  for (int r = tid; r < capacity; r += MOE_THREADS) row_token[r] = -1;
+  for (int i = tid; i < capacity / tile; i += MOE_THREADS) tile_group[i] = -1;
+  __syncthreads();
+  for (int s = tid; s < slots; s += MOE_THREADS) {
+    const int id = token_ids[s / top];
+    const int e = (id >= 0 && id < vocab) ? table[(size_t)id * top + s % top] : -1;
+    if (e >= 0 && e < experts) atomicAdd(&count[e], 1);
+  }
+  __syncthreads();
+  if (tid == 0) {
+    int at = 0;
+    for (int e = 0; e < experts; ++e) {
+      first[e] = at;
+      const int tiles = (count[e] + tile - 1) / tile;
+      for (int i = 0; i < tiles; ++i) tile_group[at / tile + i] = e;
+      at += tiles * tile;
+      count[e] = 0;  // counts again below, as the rows take their places
+    }
+  }
+  __syncthreads();
+  for (int s = tid; s < slots; s += MOE_THREADS) {
+    const int id = token_ids[s / top];
+    const int e = (id >= 0 && id < vocab) ? table[(size_t)id * top + s % top] : -1;
+    int row = -1;
+    if (e >= 0 && e < experts) {
+      row = first[e] + atomicAdd(&count[e], 1);
+      row_token[row] = s / top;
+    }
+    slot_of[s] = row;  // -1: the table names no expert of this layer; the choice adds nothing
+  }
+}
+
+extern "C" int rv_moe_route(hipStream_t stream, const int* token_ids, int num_tokens, const int* table, int vocab,
+                            int top, int experts, int tile, int capacity, int* slot_of, int* row_token,
+                            int* tile_group) {
+  RV_CHECK(num_tokens >= 0 && vocab > 0 && top > 0, "moe_route: bad sizes tokens=%d vocab=%d top=%d", num_tokens, vocab, top);
+  RV_CHECK(experts > 0 && experts <= MOE_MAX_EXPERTS, "moe_route: %d experts, at most %d are supported", experts,
+           MOE_MAX_EXPERTS);
+  RV_CHECK(tile > 0 && capacity % tile == 0 && (long long)capacity >= (long long)num_tokens * top + (long long)experts * (tile - 1),
+           "moe_route: %d rows do not hold every case of %d choices among %d experts in tiles of %d", capacity,
+           num_tokens * top, experts, tile);
+  if (num_tokens == 0) return 0;
+  moe_route_kernel<<<dim3(1), dim3(MOE_THREADS), 0, stream>>>(token_ids, num_tokens, table, vocab, top, experts, tile,
+                                                             capacity, slot_of, row_token, tile_group);
+  RV_LAUNCH_CHECK("moe_route");
+  return 0;
+}
+
+template <typename T>
+__global__ void moe_combine_kernel(const T* __restrict__ y, const int* __restrict__ slot_of, int top, float weight,
+                                   const T* __restrict__ shared, T* __restrict__ out, int width) {
+  const int t = blockIdx.x;
+  for (int i = threadIdx.x; i < width; i += blockDim.x) {
+    float acc = 0.f;
+    for (int k = 0; k < top; ++k) {
+      const int row = slot_of[(size_t)t * top + k];
+      if (row >= 0) acc += rv_to_float(y[(size_t)row * width + i]);
+    }
+    acc *= weight;
+    if (shared != nullptr) acc += rv_to_float(shared[(size_t)t * width + i]);
+    out[(size_t)t * width + i] = rv_from_float<T>(acc);
+  }
+}
+
+extern "C" int rv_moe_combine(hipStream_t stream, const void* y, const int* slot_of, int top, float weight,
+                              const void* shared, void* out, int dtype, int num_tokens, int width) {
+  RV_CHECK(num_tokens >= 0 && width > 0 && top > 0, "moe_combine: bad sizes tokens=%d width=%d top=%d", num_tokens, width, top);
+  if (num_tokens == 0) return 0;
+  dim3 grid(num_tokens), block(256);
+  if (dtype == RV_F32)
+    moe_combine_kernel<float><<<grid, block, 0, stream>>>((const float*)y, slot_of, top, weight, (const float*)shared,
+                                                          (float*)out, width);
+  else if (dtype == RV_BF16)
+    moe_combine_kernel<bf16_t><<<grid, block, 0, stream>>>((const bf16_t*)y, slot_of, top, weight,
+                                                           (const bf16_t*)shared, (bf16_t*)out, width);
+  else
+    return rv_fail("moe_combine: unsupported dtype %d", dtype);
+  RV_LAUNCH_CHECK("moe_combine");
+  return 0;
+}

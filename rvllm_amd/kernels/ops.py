@@ -202,6 +202,213 @@ def embed_gather(table: torch.Tensor, ids: torch.Tensor, scale: float, out: torc
     return out
 
 
+def embed_positions(table: torch.Tensor, pos_table: torch.Tensor, ids: torch.Tensor, positions: torch.Tensor,
+                    scale: float, out: torch.Tensor) -> torch.Tensor:
+    """out[t] = table[ids[t]] * scale + pos_table[positions[t]], added in 32-bit."""
+    _gpu(table, pos_table, ids, positions, out)
+    _i32(ids, positions)
+    vocab, hidden = table.shape
+    n = out.shape[0]
+    _need(pos_table.dim() == 2 and pos_table.shape[1] == hidden and pos_table.dtype == table.dtype,
+          "embed_positions: the position table must have the token table's width and type")
+    _need(out.shape == (n, hidden) and ids.numel() >= n and positions.numel() >= n,
+          f"embed_positions: out is {tuple(out.shape)}, ids and positions must cover its rows")
+    _check(library().rv_embed_positions(_stream(), _ptr(table), _ptr(pos_table), _dt(table), _ptr(ids), _ptr(positions),
+                                        _ptr(out), _dt(out), _c_int(n), _c_int(hidden), _c_int(vocab),
+                                        _c_int(pos_table.shape[0]), _c_float(scale)))
+    return out
+
+
+def scalar_rmsnorm(x: torch.Tensor, gain: torch.Tensor, eps: float, out_dtype: Optional[torch.dtype] = None,
+                   out: Optional[torch.Tensor] = None, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Row-wise x * rsqrt(mean(x^2) + eps) * gain with one number as the gain.  ``x`` may be the 32-bit residual
+    stream of a bf16 model: the result then has ``out_dtype``.  ``rows`` as in ``rmsnorm``."""
+    _gpu(x, gain, out, rows)
+    _need(x.dim() == 2, "scalar_rmsnorm: a matrix is expected")
+    _need(gain.numel() == 1 and gain.dtype in _DT, "scalar_rmsnorm: the gain is one number")
+    width = x.shape[1]
+    if rows is not None:
+        _i32(rows)
+    n_rows = x.shape[0] if rows is None else rows.numel()
+    if out is None:
+        out = torch.empty((n_rows, width), dtype=out_dtype or x.dtype, device=x.device)
+    _need(out.shape == (n_rows, width), "scalar_rmsnorm: bad out")
+    _check(library().rv_scalar_rmsnorm(_stream(), _ptr(x), _dt(x), _ptr(rows), _ptr(gain),
+                                       _c_int(gain.dtype == torch.float32), _ptr(out), _dt(out), _c_int(n_rows),
+                                       _c_int(width), _c_float(eps)))
+    return out
+
+
+def residual_mix(x: torch.Tensor, mixer_branch, ff_branch, mult: float, history: Optional[torch.Tensor] = None,
+                 terms: int = 0, depth_weights: Optional[torch.Tensor] = None, seed_history: bool = False,
+                 next_gain: Optional[torch.Tensor] = None, next_eps: float = 0.0,
+                 next_dtype: Optional[torch.dtype] = None) -> Optional[torch.Tensor]:
+    """The 32-bit residual stream ``x [rows, width]`` takes a layer's two branches, in place:
+    X = x + mult * (mixer_branch + ff_branch); with ``history`` (float32 ``[slots, rows, width]``) X is kept as
+    entry ``terms - 1`` and x becomes sum_j depth_weights[j] * history[j] over the first ``terms`` entries
+    (``seed_history``: entry 0 is x as it came in); otherwise x becomes X.  With ``next_gain`` also returns
+    ``scalar_rmsnorm`` of the new x in ``next_dtype``.  A branch is a tensor of the activations' type, unreduced
+    ``SlicedSums``, or (the feed-forward's) None."""
+    _gpu(x, history, depth_weights, next_gain)
+    _need(x.dtype == torch.float32 and x.dim() == 2, "residual_mix: the residual stream is a 32-bit matrix")
+    rows, width = x.shape
+    aptr, a_slices, a_stride, a_rows, a_width, a_dtype = _branch_args(mixer_branch, "residual_mix")
+    _need((a_rows, a_width) == (rows, width), "residual_mix: the mixer's branch must match the residual stream")
+    fptr, f_slices, f_stride = None, 0, 0
+    if ff_branch is not None:
+        fptr, f_slices, f_stride, f_rows, f_width, f_dtype = _branch_args(ff_branch, "residual_mix")
+        _need((f_rows, f_width) == (rows, width) and f_dtype == a_dtype,
+              "residual_mix: the feed-forward's branch must match the mixer's")
+    stride = 0
+    if history is not None:
+        _need(history.dtype == torch.float32 and history.dim() == 3 and tuple(history.shape[1:]) == (rows, width)
+              and 2 <= terms <= history.shape[0], "residual_mix: the history must be 32-bit [slots >= terms, rows, width]")
+        _need(depth_weights is not None and depth_weights.numel() == terms and depth_weights.dtype in _DT,
+              f"residual_mix: {terms} depth weights expected")
+        stride = history.stride(0)
+    nxt = None
+    if next_gain is not None:
+        _need(next_gain.numel() == 1 and next_gain.dtype in _DT, "residual_mix: the next norm's gain is one number")
+        nxt = torch.empty((rows, width), dtype=next_dtype or a_dtype, device=x.device)
+        _need(nxt.dtype == a_dtype, "residual_mix: the next norm's output has the branches' type")
+    _check(library().rv_residual_mix(
+        _stream(), _ptr(x), aptr, _c_int(a_slices), _c_ll(a_stride), fptr, _c_int(f_slices), _c_ll(f_stride),
+        _c_float(mult), _ptr(history), _c_ll(stride), _c_int(terms), _c_int(int(seed_history)), _ptr(depth_weights),
+        _c_int(depth_weights is not None and depth_weights.dtype == torch.float32), _ptr(next_gain),
+        _c_int(next_gain is not None and next_gain.dtype == torch.float32), _ptr(nxt), _c_float(next_eps),
+        _DT[a_dtype], _c_int(rows), _c_int(width)))
+    return nxt
+
+
+def latent_norm_write(raw: torch.Tensor, col0: int, rank: int, weight: torch.Tensor, eps: float, offset: float,
+                      positions: torch.Tensor, token_req: torch.Tensor, block_table: torch.Tensor,
+                      k_pages: torch.Tensor, v_pages: torch.Tensor) -> None:
+    """Columns ``col0 .. col0 + rank`` of the rows of ``raw``, RMS-normed with ``weight``, into the one-head cache
+    ``k_pages`` / ``v_pages`` at each token's position."""
+    _gpu(raw, weight, positions, token_req, block_table, k_pages, v_pages)
+    _i32(positions, token_req, block_table)
+    n = raw.shape[0]
+    num_pages, nkv, page_size, hd = _cache_geometry(k_pages, v_pages, "latent_norm_write")
+    _need(nkv == 1 and hd == rank, f"latent_norm_write: the cache must hold one head of {rank} dimensions")
+    _need(raw.dim() == 2 and 0 <= col0 and col0 + rank <= raw.shape[1], "latent_norm_write: columns outside the rows")
+    _need(k_pages.dtype == raw.dtype and v_pages.dtype == raw.dtype, "latent_norm_write: cache dtype differs")
+    _need(weight.shape == (rank,) and weight.dtype in _DT, f"latent_norm_write: the norm's weight must hold {rank} numbers")
+    _need(positions.numel() >= n and token_req.numel() >= n, "latent_norm_write: positions/token_req too short")
+    _check(library().rv_latent_norm_write(
+        _stream(), _ptr(raw), _c_ll(raw.stride(0)), _c_int(col0), _ptr(weight), _c_int(weight.dtype == torch.float32),
+        _c_float(eps), _c_float(offset), _ptr(positions), _ptr(token_req), _ptr(block_table),
+        _c_int(block_table.shape[1]), _ptr(k_pages), _ptr(v_pages), _c_int(page_size), _c_int(num_pages), _c_int(rank),
+        _c_int(n), _dt(raw)))
+
+
+def gemm_heads(a: torch.Tensor, a_col0: int, w: torch.Tensor, out: Optional[torch.Tensor] = None,
+               gate: Optional[torch.Tensor] = None, gate_col0: int = 0) -> torch.Tensor:
+    """One product a head, side by side: ``w`` is ``[heads, N, K]``; head h multiplies columns
+    ``a_col0 + h K .. + K`` of the rows of ``a`` and fills columns ``h N .. + N`` of ``out [rows, heads N]``.
+    With ``gate`` the result is multiplied by sigmoid of the columns ``gate_col0 + ...`` of the rows of ``gate``,
+    laid out like ``out``."""
+    _need(a.is_cuda and w.is_cuda and a.dim() == 2 and w.dim() == 3 and w.is_contiguous() and a.stride(1) == 1,
+          "gemm_heads: rows of inputs and [heads, N, K] matrices on the GPU expected")
+    heads, n, k = w.shape
+    m = a.shape[0]
+    _need(a_col0 >= 0 and a_col0 + heads * k <= a.shape[1], "gemm_heads: the heads' inputs lie outside the rows")
+    _need(a.dtype == w.dtype and a.dtype in _DT, "gemm_heads: inputs and matrices of one type, float32 or bfloat16")
+    if out is None:
+        out = torch.empty((m, heads * n), dtype=a.dtype, device=a.device)
+    _need(out.shape == (m, heads * n) and out.dtype == a.dtype and out.is_contiguous(), "gemm_heads: bad out")
+    gptr, ldg = None, 0
+    if gate is not None:
+        _need(gate.is_cuda and gate.dim() == 2 and gate.stride(1) == 1 and gate.dtype == out.dtype
+              and gate.shape[0] == m and 0 <= gate_col0 and gate_col0 + heads * n <= gate.shape[1],
+              "gemm_heads: the gate must hold the output's columns in its rows")
+        gptr, ldg = gate.data_ptr() + gate_col0 * gate.element_size(), gate.stride(0)
+    _check(library().rv_gemm_groups_plain(
+        _stream(), a.data_ptr() + a_col0 * a.element_size(), _dt(a), _ptr(w), _dt(w), _ptr(out), _dt(out), None, None,
+        _c_int(heads), _c_int(m), _c_int(n), _c_int(k), _c_ll(a.stride(0)), _c_ll(k), _c_ll(out.stride(0)), _c_ll(k),
+        _c_ll(n * k), _c_ll(n), gptr, _c_ll(ldg)))
+    return out
+
+
+MOE_TILE_ROWS = 64  # rows of one expert that a block of the grouped product takes
+
+
+def moe_capacity(num_tokens: int, top: int, experts: int, tile: int = MOE_TILE_ROWS) -> int:
+    """Sorted rows that hold every routing of ``num_tokens * top`` choices: each expert's rows start a tile."""
+    return -(-(num_tokens * top + experts * (tile - 1)) // tile) * tile
+
+
+def moe_route(token_ids: torch.Tensor, num_tokens: int, table: torch.Tensor, experts: int,
+              tile: int = MOE_TILE_ROWS) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """Sorts the step's (token, choice) pairs by the expert that ``table [vocab, top]`` gives the token's id.
+    Returns (slot_of ``[tokens * top]``: the sorted row of each pair; row_token ``[capacity]``: the token of each
+    sorted row, -1 for filling rows; tile_group ``[capacity / tile]``: the expert of each tile of rows, or -1)."""
+    _gpu(token_ids, table)
+    _i32(token_ids, table)
+    _need(table.dim() == 2 and token_ids.numel() >= num_tokens, "moe_route: a table [vocab, top] and the step's ids")
+    vocab, top = table.shape
+    capacity = moe_capacity(num_tokens, top, experts, tile)
+    slot_of = torch.empty(num_tokens * top, dtype=torch.int32, device=table.device)
+    row_token = torch.empty(capacity, dtype=torch.int32, device=table.device)
+    tile_group = torch.empty(capacity // tile, dtype=torch.int32, device=table.device)
+    _check(library().rv_moe_route(_stream(), _ptr(token_ids), _c_int(num_tokens), _ptr(table), _c_int(vocab),
+                                  _c_int(top), _c_int(experts), _c_int(tile), _c_int(capacity), _ptr(slot_of),
+                                  _ptr(row_token), _ptr(tile_group)))
+    return slot_of, row_token, tile_group
+
+
+def gemm_experts(a: torch.Tensor, w: torch.Tensor, tile_group: torch.Tensor, row_index: Optional[torch.Tensor] = None,
+                 out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``out[r] = a[row_index[r]] @ w[tile_group[r // tile]]^T`` for the sorted rows of ``moe_route``; ``w`` is
+    ``[experts, N, K]``.  Without ``row_index`` the rows of ``a`` are the sorted rows themselves.  Rows of tiles
+    without an expert are left as they are."""
+    _gpu(a, w, tile_group, row_index, out)
+    _i32(tile_group)
+    _need(a.dim() == 2 and w.dim() == 3 and a.dtype == w.dtype and a.dtype in _DT and a.shape[1] == w.shape[2],
+          "gemm_experts: rows [*, K] against matrices [experts, N, K] of one type expected")
+    m = tile_group.numel() * MOE_TILE_ROWS
+    if row_index is not None:
+        _i32(row_index)
+        _need(row_index.numel() == m, "gemm_experts: one source row for every sorted row")
+    else:
+        _need(a.shape[0] == m, "gemm_experts: the rows must be the sorted rows")
+    _, n, k = w.shape
+    if out is None:
+        out = torch.empty((m, n), dtype=a.dtype, device=a.device)
+    _need(out.shape == (m, n) and out.dtype == a.dtype, "gemm_experts: bad out")
+    _check(library().rv_gemm_groups_plain(
+        _stream(), _ptr(a), _dt(a), _ptr(w), _dt(w), _ptr(out), _dt(out), _ptr(row_index), _ptr(tile_group), _c_int(0),
+        _c_int(m), _c_int(n), _c_int(k), _c_ll(a.stride(0)), _c_ll(k), _c_ll(n), _c_ll(0), _c_ll(n * k), _c_ll(0),
+        None, _c_ll(0)))
+    return out
+
+
+def moe_combine(y: torch.Tensor, slot_of: torch.Tensor, top: int, weight: float, num_tokens: int,
+                shared: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out[t] = weight * sum_k y[slot_of[t * top + k]] (+ shared[t])."""
+    _gpu(y, slot_of, shared)
+    _i32(slot_of)
+    width = y.shape[1]
+    _need(slot_of.numel() == num_tokens * top, "moe_combine: one sorted row for every choice")
+    _need(shared is None or (shared.shape == (num_tokens, width) and shared.dtype == y.dtype),
+          "moe_combine: the shared expert's output must match")
+    out = torch.empty((num_tokens, width), dtype=y.dtype, device=y.device)
+    _check(library().rv_moe_combine(_stream(), _ptr(y), _ptr(slot_of), _c_int(top), _c_float(weight), _ptr(shared),
+                                    _ptr(out), _dt(out), _c_int(num_tokens), _c_int(width)))
+    return out
+
+
+def clamped_glu(gate_up: torch.Tensor, limit: float, alpha: float) -> torch.Tensor:
+    """g = min(gate, limit), u = clamp(up, -limit, limit): out = g * sigmoid(alpha g) * (u + 1); gates and ups lie in
+    the halves of a row of ``gate_up [rows, 2 I]``."""
+    _gpu(gate_up)
+    _need(gate_up.dim() == 2 and gate_up.shape[1] % 2 == 0, "clamped_glu: rows of gates and ups expected")
+    rows, inter = gate_up.shape[0], gate_up.shape[1] // 2
+    out = torch.empty((rows, inter), dtype=gate_up.dtype, device=gate_up.device)
+    _check(library().rv_clamped_glu(_stream(), _ptr(gate_up), _ptr(out), _dt(out), _c_int(rows), _c_int(inter),
+                                    _c_float(limit), _c_float(alpha)))
+    return out
+
+
 def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, offset: float,
             out: Optional[torch.Tensor] = None, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Row-wise RMSNorm.  With ``rows`` (int32 indices into the rows of a 2-d
@@ -397,10 +604,20 @@ def qk_norm_rope_kv_write(qkv, q_out: torch.Tensor, q_weight: Optional[torch.Ten
 VALUES_BY_PAGE_MIN_PORTION = 16
 
 
+def _check_sinks(sinks: Optional[torch.Tensor], num_q_heads: int) -> None:
+    if sinks is not None:
+        _gpu(sinks)
+        _need(sinks.dtype == torch.float32 and sinks.shape == (num_q_heads,),
+              f"attention: the sinks must be {num_q_heads} 32-bit numbers, one a query head")
+
+
 def paged_attention_generic(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, block_table: torch.Tensor,
                             positions: torch.Tensor, token_req: torch.Tensor, out: torch.Tensor, num_q_heads: int,
-                            scale: float, window: Optional[int]) -> torch.Tensor:
+                            scale: float, window: Optional[int], sinks: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``sinks``: one 32-bit number a query head; head h's sum of exponentials then has one more term
+    e^(sinks[h]), with no key and no value."""
     _gpu(q, k_pages, v_pages, block_table, positions, token_req, out)
+    _check_sinks(sinks, num_q_heads)
     _i32(block_table, positions, token_req)
     n = q.shape[0]
     num_pages, nkv, page_size, hd = _cache_geometry(k_pages, v_pages, "attention")
@@ -411,21 +628,23 @@ def paged_attention_generic(q: torch.Tensor, k_pages: torch.Tensor, v_pages: tor
     _check(library().rv_paged_attention_generic(
         _stream(), _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(block_table), _c_int(block_table.shape[1]),
         _ptr(positions), _ptr(token_req), _ptr(out), _dt(q), _c_int(n), _c_int(num_q_heads), _c_int(nkv), _c_int(hd),
-        _c_int(page_size), _c_int(num_pages), _c_int(window or 0), _c_float(scale)))
+        _c_int(page_size), _c_int(num_pages), _c_int(window or 0), _c_float(scale), _ptr(sinks)))
     return out
 
 
 def paged_attention(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, block_table: torch.Tensor, step,
-                    out: torch.Tensor, num_q_heads: int, scale: float, window: Optional[int]) -> torch.Tensor:
+                    out: torch.Tensor, num_q_heads: int, scale: float, window: Optional[int],
+                    sinks: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Attention of the step's tokens over the cache; picks the kernel.
 
     The 32-bit path always runs the generic kernel.  bf16 runs the
     matrix-core kernel where it covers the head size and grouping, else the
     generic one."""
     if q.dtype == torch.bfloat16 and mfma_attention_covers(k_pages, v_pages, num_q_heads):
-        return paged_attention_mfma(q, k_pages, v_pages, block_table, step, out, num_q_heads, scale, window)
+        return paged_attention_mfma(q, k_pages, v_pages, block_table, step, out, num_q_heads, scale, window,
+                                    sinks=sinks)
     return paged_attention_generic(q, k_pages, v_pages, block_table, step.positions, step.token_req, out,
-                                   num_q_heads, scale, window)
+                                   num_q_heads, scale, window, sinks)
 
 
 MFMA_ATTENTION_MAX_HEAD_DIM = 256
@@ -660,7 +879,8 @@ def paged_attention_mfma(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.
                          step, out: torch.Tensor, num_q_heads: int, scale: float, window: Optional[int],
                          splits: Optional[tuple[int, int]] = None, prefill_kernel: Optional[bool] = None,
                          in_block: Optional[bool] = None,
-                         prefill_pieces: Optional[tuple[int, int]] = None) -> torch.Tensor:
+                         prefill_pieces: Optional[tuple[int, int]] = None,
+                         sinks: Optional[torch.Tensor] = None) -> torch.Tensor:
     """bf16 attention on the matrix cores.  ``splits`` = (number, keys per
     split) overrides the plan, ``prefill_kernel`` the choice of kernel,
     ``in_block`` whether a tile's splits are merged inside one block and
@@ -669,6 +889,7 @@ def paged_attention_mfma(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.
     every path)."""
     _gpu(q, k_pages, v_pages, block_table, out)
     _i32(block_table)
+    _check_sinks(sinks, num_q_heads)
     n = q.shape[0]
     num_pages, nkv, page_size, hd = _cache_geometry(k_pages, v_pages, "attention")
     _need(q.dtype == torch.bfloat16 and k_pages.dtype == torch.bfloat16 and v_pages.dtype == torch.bfloat16,
@@ -713,7 +934,7 @@ def paged_attention_mfma(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.
                      _c_int(block_table.shape[1]), _ptr(step.q_start), _ptr(step.chunk_start), _ptr(out), _c_int(n),
                      _c_int(step.num_requests), _c_int(tiles), _c_int(num_q_heads), _c_int(nkv), _c_int(hd),
                      _c_int(page_size), _c_int(num_pages), _c_int(window or 0), _c_int(portion_min), _c_float(scale),
-                     _c_int(piece_max), _c_int(pieces_max), _ptr(part)))
+                     _c_int(piece_max), _c_int(pieces_max), _ptr(part), _ptr(sinks)))
     if shortest_rest > 0:
         tiles, num_splits, split_len = plan_attention_splits(step.num_requests, shortest_rest, step.max_context, nkv,
                                                              group, window, hd, attention_wave_slots(hd))
@@ -742,7 +963,7 @@ def paged_attention_mfma(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.
                      _ptr(out), _ptr(part_o), _ptr(part_ml), _c_int(n), _c_int(step.num_requests), _c_int(tiles),
                      _c_int(num_q_heads), _c_int(nkv), _c_int(hd), _c_int(page_size), _c_int(num_pages),
                      _c_int(window or 0), _c_int(num_splits), _c_int(split_len),
-                     _c_int(portion_min - 1 if use_prefill else 0), _c_int(block_cols), _c_float(scale)))
+                     _c_int(portion_min - 1 if use_prefill else 0), _c_int(block_cols), _c_float(scale), _ptr(sinks)))
     return out
 
 

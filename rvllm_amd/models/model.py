@@ -105,7 +105,8 @@ class DecoderModel:
         """Runs the step's tokens; returns float32 logits ``[wanted rows, vocab]``.
 
         ``caches[i]`` is the cache view of layer i."""
-        x = torch.empty((step.num_tokens, self.spec.hidden_size), dtype=self.dtype, device=self.device)
+        x = torch.empty((step.num_tokens, self.spec.hidden_size), device=self.device,
+                        dtype=torch.float32 if self.spec.residual_float32 else self.dtype)
         self.embedding.forward(step, x)
         schedule = self.spec.schedule
         entered = None

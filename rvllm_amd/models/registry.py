@@ -1,7 +1,8 @@
 """The one registry from an architecture's name to its model.
 
 config.json's ``architectures[0]`` picks the entry, as in the reference
-(v3/crates/rvllm-core/src/config/model.rs:14-36,71-80).  An entry knows how to
+(v3/crates/rvllm-core/src/config/model.rs:14-36,71-80); a file without that
+list may name its design in a string ``architecture``.  An entry knows how to
 read its configuration, how its checkpoints name their tensors, and how to
 turn both into a ``ModelSpec``; everything else is shared.
 """
@@ -92,9 +93,11 @@ def read_config_file(model_dir: str | os.PathLike) -> tuple[dict, str]:
 
 def architecture_of(doc: dict, source: str = "config.json") -> Architecture:
     archs = doc.get("architectures")
-    if not (isinstance(archs, list) and archs and isinstance(archs[0], str)):
-        raise ConfigError(source, ["missing or invalid required field architectures[0]"])
-    return get_architecture(archs[0], source)
+    if isinstance(archs, list) and archs and isinstance(archs[0], str):
+        return get_architecture(archs[0], source)
+    if archs is None and isinstance(doc.get("architecture"), str):
+        return get_architecture(doc["architecture"], source)
+    raise ConfigError(source, ["missing or invalid required field architectures[0] (or architecture)"])
 
 
 def load_config(model_dir: str | os.PathLike) -> tuple[Architecture, Any]:

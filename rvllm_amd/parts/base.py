@@ -34,6 +34,11 @@ class ParamSpec:
     integer: bool = False
 
 
+def tensor_path(prefix: str, name: str) -> str:
+    """``name`` under ``prefix``; a checkpoint that keeps its tensors under no prefix has the empty one."""
+    return f"{prefix}.{name}" if prefix else name
+
+
 class Part:
     """Base of every part.
 

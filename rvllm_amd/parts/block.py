@@ -11,6 +11,17 @@ v3/crates/rvllm-runtime/src/gemma4_layer_exec.rs:1-28):
 A block may hand the next block its entry norm already applied (``then``),
 which lets the kernel that adds the feed-forward branch also write the next
 layer's normed input.
+
+``parallel``: one norm, both branches read its output, and their sum is added
+with a multiplier; the residual stream is 32-bit whatever the activations' type:
+
+    h = norm(x);  X = x + residual_mult * (mixer(h) + ff(h))
+
+With ``depth_average`` = {"name", "terms", "slots"} what goes on to the next
+layer is a learned average over depth, x = sum_j w[j] * X_j over the first
+``terms`` of: the first layer's input and every layer's X so far (``slots`` in
+all; the tensor ``<layer>.<name>`` holds the ``terms`` weights).  The X_j of a
+step live in ``step.shared`` and end with it.
 """
 
 from __future__ import annotations
@@ -19,7 +30,9 @@ from typing import Optional
 
 import torch
 
-from .base import Block, Norm, ParamSpec
+from ..kernels import ops
+from .base import Block, Norm, ParamSpec, tensor_path
+from .norm import ScalarRMSNorm
 from .registry import BLOCKS, FEED_FORWARDS, MIXERS, NORMS
 from .spec import LayerSpec, PartSpec
 
@@ -58,4 +71,68 @@ class SandwichBlock(Block):
         return self.norm_post_ff.add_into(f, x, then=then)
 
 
+class ParallelBlock(Block):
+    HISTORY = "parallel_block.depth_history"  # key in step.shared: (the X_j, how many are written)
+
+    def __init__(self, spec: PartSpec, *, layer: LayerSpec, hidden_size: int):
+        self.hidden_size = hidden_size
+        self.residual_mult = float(spec.get("residual_mult", 1.0))
+        self.norm_name = str(spec.get("norm_name", "norm"))
+        depth = spec.get("depth_average")
+        self.depth = None if depth is None else {"name": str(depth["name"]), "terms": int(depth["terms"]),
+                                                 "slots": int(depth["slots"])}
+        if self.depth is not None and not 2 <= self.depth["terms"] <= self.depth["slots"]:
+            raise ValueError(f"a depth average over {self.depth['terms']} of {self.depth['slots']} streams")
+        self.mixer = MIXERS.build(layer.mixer, hidden_size=hidden_size)
+        self.feed_forward = FEED_FORWARDS.build(layer.feed_forward, hidden_size=hidden_size)
+        self.norm = NORMS.build(layer.norm, width=hidden_size, name=self.norm_name)
+        self.depth_weights: Optional[torch.Tensor] = None
+
+    def parts(self):
+        return (self.mixer, self.feed_forward, self.norm)
+
+    def param_specs(self, prefix: str) -> list[ParamSpec]:
+        specs = [s for part in self.parts() for s in part.param_specs(prefix)]
+        if self.depth is not None:
+            specs.append(ParamSpec(tensor_path(prefix, self.depth["name"]), (self.depth["terms"],),
+                                   init=("normal_about", 1.0 / self.depth["terms"], 0.05)))
+        return specs
+
+    def bind(self, tensors, prefix, device, dtype) -> None:
+        for part in self.parts():
+            part.bind(tensors, prefix, device, dtype)
+        if self.depth is not None:  # averaged in 32-bit
+            self.depth_weights = tensors[tensor_path(prefix, self.depth["name"])].to(
+                device=device, dtype=torch.float32).contiguous()
+
+    def entry_norm(self) -> Optional[Norm]:
+        return self.norm
+
+    def forward(self, x: torch.Tensor, step, cache, entered: Optional[torch.Tensor] = None,
+                then: Optional[Norm] = None) -> Optional[torch.Tensor]:
+        h = entered if entered is not None else self.norm.forward(x)
+        a = self.mixer.forward(h, step, cache)
+        f = self.feed_forward.forward(h, step)
+        history, terms, seed = None, 0, False
+        if self.depth is not None:
+            terms = self.depth["terms"]
+            kept = step.shared.get(self.HISTORY)
+            if kept is None:  # the first layer of the step: its input is the first of the streams
+                kept = [torch.empty((self.depth["slots"], *x.shape), dtype=torch.float32, device=x.device), 1]
+                step.shared[self.HISTORY] = kept
+                seed = True
+            history = kept[0]
+            if kept[1] != terms - 1:
+                raise ValueError(f"a depth average over {terms} streams, but the step has written {kept[1]}")
+            kept[1] = terms
+        fused = isinstance(then, ScalarRMSNorm)
+        nxt = ops.residual_mix(x, a, f, self.residual_mult, history, terms, self.depth_weights, seed,
+                               then.gain if fused else None, then.eps if fused else 0.0,
+                               then.out_dtype if fused else None)
+        if then is not None and not fused:
+            return then.forward(x)
+        return nxt
+
+
 BLOCKS.register("sandwich", SandwichBlock)
+BLOCKS.register("parallel", ParallelBlock)

@@ -18,7 +18,7 @@ from typing import Optional
 import torch
 
 from ..kernels import ops
-from .base import Embedding, Head, ParamSpec
+from .base import Embedding, Head, ParamSpec, tensor_path
 from .linear import decode_weight, linear
 from .registry import EMBEDDINGS, HEADS
 from .spec import PartSpec
@@ -43,6 +43,36 @@ class ScaledEmbedding(Embedding):
 
     def forward(self, step, out: torch.Tensor) -> torch.Tensor:
         return ops.embed_gather(self.table, step.token_ids, self.scale, out)
+
+
+class PositionalEmbedding(Embedding):
+    """x[t] = table[id[t]] * scale + positions[p[t]]: a learned vector for every position is added to the token's,
+    in 32-bit.  Parameters: ``scale`` (1 if absent), ``max_position`` (rows of the position table), ``name`` and
+    ``position_name`` (the two tables' names under the model's prefix) and ``suffix`` (what follows a name;
+    ``.weight`` if absent)."""
+
+    def __init__(self, spec: PartSpec, *, hidden_size: int, vocab_size: int):
+        self.hidden_size = hidden_size
+        self.vocab_size = vocab_size
+        self.scale = float(spec.get("scale", 1.0))
+        self.max_position = int(spec["max_position"])
+        self.name = str(spec.get("name", "embed_tokens"))
+        self.position_name = str(spec.get("position_name", "embed_positions"))
+        self.suffix = str(spec.get("suffix", ".weight"))
+        self.table: Optional[torch.Tensor] = None
+        self.positions: Optional[torch.Tensor] = None
+
+    def param_specs(self, prefix: str) -> list[ParamSpec]:
+        return [ParamSpec(tensor_path(prefix, self.name) + self.suffix, (self.vocab_size, self.hidden_size)),
+                ParamSpec(tensor_path(prefix, self.position_name) + self.suffix, (self.max_position, self.hidden_size))]
+
+    def bind(self, tensors, prefix, device, dtype) -> None:
+        self.table = tensors[tensor_path(prefix, self.name) + self.suffix].to(device=device, dtype=dtype).contiguous()
+        self.positions = tensors[tensor_path(prefix, self.position_name) + self.suffix].to(
+            device=device, dtype=dtype).contiguous()
+
+    def forward(self, step, out: torch.Tensor) -> torch.Tensor:
+        return ops.embed_positions(self.table, self.positions, step.token_ids, step.positions, self.scale, out)
 
 
 class LMHead(Head):
@@ -83,4 +113,5 @@ class LMHead(Head):
 
 
 EMBEDDINGS.register("scaled_embedding", ScaledEmbedding)
+EMBEDDINGS.register("positional_embedding", PositionalEmbedding)
 HEADS.register("lm_head", LMHead)

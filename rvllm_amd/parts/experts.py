@@ -1,0 +1,112 @@
+"""A mixture of experts: each token's feed-forward is the weighted sum of a few small gated feed-forwards.
+
+Which experts a token uses is the router's matter.  ``token_table``: a stored
+integer table ``[vocab, top]`` gives each token id its ``top`` experts (the
+entries of a row differ), each with weight 1 / top; nothing is learned from
+the activations.  The step's (token, choice) pairs are sorted by expert on the
+device (``ops.moe_route``), each expert's rows are multiplied against its own
+matrices in one launch for all experts (``ops.gemm_experts``), and the results
+return to their tokens (``ops.moe_combine``): no launch depends on which
+experts the tokens chose, so a step can be replayed from a graph.
+
+An expert computes down(act(gate(x), up(x))) without biases.  ``activation``:
+``clamped_glu`` with ``limit`` and ``alpha``: g = min(gate, limit), u =
+clamp(up, -limit, limit), act = g * sigmoid(alpha g) * (u + 1).
+``shared`` (optional: ``intermediate_size``, ``limit``, ``alpha``) is one more
+expert of the same form that every token uses with weight 1.
+
+``names``: ``expert`` (a pattern with ``{}`` for the expert's number),
+``table``, ``shared`` under the layer's prefix; ``gate``, ``up``, ``down``
+under an expert's name.
+"""
+
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from ..kernels import ops
+from .base import FeedForward, ParamSpec
+from .linear import decode_weight, linear, tensor_names
+from .registry import FEED_FORWARDS
+from .spec import PartSpec
+
+
+class RoutedExperts(FeedForward):
+    NAMES = {"expert": "mlp.e{}", "table": "mlp.table", "shared": "mlp.shared", "gate": "gate", "up": "up",
+             "down": "down"}
+    ROUTERS = ("token_table",)
+    ACTIVATIONS = ("clamped_glu",)
+
+    def __init__(self, spec: PartSpec, *, hidden_size: int):
+        self.hidden_size = int(hidden_size)
+        self.num_experts = int(spec["experts"])
+        self.top = int(spec["top"])
+        self.intermediate_size = int(spec["intermediate_size"])
+        self.router = str(spec.get("router", "token_table"))
+        self.activation = str(spec.get("activation", "clamped_glu"))
+        if self.router not in self.ROUTERS:
+            raise ValueError(f"unknown router {self.router!r}; known: {self.ROUTERS}")
+        if self.activation not in self.ACTIVATIONS:
+            raise ValueError(f"unknown expert activation {self.activation!r}; known: {self.ACTIVATIONS}")
+        if not 1 <= self.top <= self.num_experts:
+            raise ValueError(f"{self.top} of {self.num_experts} experts a token")
+        self.vocab_size = int(spec["vocab_size"])
+        self.limit = float(spec["limit"])
+        self.alpha = float(spec.get("alpha", 1.702))
+        shared = spec.get("shared")
+        self.shared = None if shared is None else {
+            "intermediate_size": int(shared["intermediate_size"]), "limit": float(shared["limit"]),
+            "alpha": float(shared.get("alpha", self.alpha))}
+        self.names = tensor_names(self.NAMES, spec.get("names"))
+        self.table = self.w_gate_up = self.w_down = self.shared_gate_up = self.shared_down = None
+
+    # ---- weights -----------------------------------------------------
+    def _expert_names(self, prefix: str, e: Optional[int]) -> dict:
+        base = f"{prefix}.{self.names['shared']}" if e is None else f"{prefix}.{self.names['expert'].format(e)}"
+        return {role: f"{base}.{self.names[role]}" for role in ("gate", "up", "down")}
+
+    def param_specs(self, prefix: str) -> list[ParamSpec]:
+        H, I = self.hidden_size, self.intermediate_size
+        specs = []
+        for e in range(self.num_experts):
+            at = self._expert_names(prefix, e)
+            specs += [ParamSpec(at["gate"], (I, H)), ParamSpec(at["up"], (I, H)), ParamSpec(at["down"], (H, I))]
+        specs.append(ParamSpec(f"{prefix}.{self.names['table']}", (self.vocab_size, self.top),
+                               init=("distinct", self.num_experts), integer=True))
+        if self.shared is not None:
+            at, S = self._expert_names(prefix, None), self.shared["intermediate_size"]
+            specs += [ParamSpec(at["gate"], (S, H)), ParamSpec(at["up"], (S, H)), ParamSpec(at["down"], (H, S))]
+        return specs
+
+    def bind(self, tensors, prefix, device, dtype) -> None:
+        def get(name):
+            return tensors[name].to(device=device, dtype=dtype)
+
+        ats = [self._expert_names(prefix, e) for e in range(self.num_experts)]
+        # [experts, 2 I, H]: an expert's gates, then its ups; [experts, H, I]
+        self.w_gate_up = torch.stack([torch.cat([get(at["gate"]), get(at["up"])], dim=0) for at in ats]).contiguous()
+        self.w_down = torch.stack([get(at["down"]) for at in ats]).contiguous()
+        self.table = tensors[f"{prefix}.{self.names['table']}"].to(device=device, dtype=torch.int32).contiguous()
+        if self.shared is not None:
+            at = self._expert_names(prefix, None)
+            self.shared_gate_up = decode_weight(torch.cat([get(at["gate"]), get(at["up"])], dim=0).contiguous(),
+                                                self.tiled_weights)
+            self.shared_down = decode_weight(get(at["down"]).contiguous(), self.tiled_weights)
+
+    # ---- run ---------------------------------------------------------
+    def forward(self, x: torch.Tensor, step) -> torch.Tensor:
+        n = x.shape[0]
+        shared = None
+        if self.shared is not None:
+            act = ops.clamped_glu(linear(x, self.shared_gate_up), self.shared["limit"], self.shared["alpha"])
+            shared = linear(act, self.shared_down)
+        slot_of, row_token, tile_group = ops.moe_route(step.token_ids, n, self.table, self.num_experts)
+        gate_up = ops.gemm_experts(x, self.w_gate_up, tile_group, row_index=row_token)
+        act = ops.clamped_glu(gate_up, self.limit, self.alpha)
+        y = ops.gemm_experts(act, self.w_down, tile_group)
+        return ops.moe_combine(y, slot_of, self.top, 1.0 / self.top, n, shared)
+
+
+FEED_FORWARDS.register("routed_experts", RoutedExperts)

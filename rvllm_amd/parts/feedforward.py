@@ -10,6 +10,10 @@ few rows can apply the activation itself); the activation is a parameter
 layer's prefix, without ``.weight`` (the Gemma names if absent); a role
 ``gate_up`` names one stored matrix that holds the gate rows and then the up
 rows.  ``bias`` lists the projections that have a ``.bias`` (True: all).
+``weight_suffix`` and ``bias_suffix`` are what a projection's name is followed
+by (``.weight`` and ``.bias`` if absent).
+
+``none`` is the feed-forward of a layer that has none: it adds nothing.
 """
 
 from __future__ import annotations
@@ -33,6 +37,8 @@ class GatedMLP(FeedForward):
         if self.activation not in ops.ACTIVATIONS:
             raise ValueError(f"unknown activation {self.activation!r}; known: {sorted(ops.ACTIVATIONS)}")
         self.names = tensor_names(self.NAMES, spec.get("names"))
+        self.w_suffix = str(spec.get("weight_suffix", ".weight"))
+        self.b_suffix = str(spec.get("bias_suffix", ".bias"))
         inter = self.intermediate_size
         self.stored = {"gate_up": 2 * inter} if "gate_up" in self.names else {"gate": inter, "up": inter}
         self.bias = bias_roles(spec.get("bias"), [*self.stored, "down"])
@@ -41,41 +47,42 @@ class GatedMLP(FeedForward):
 
     def param_specs(self, prefix: str) -> list[ParamSpec]:
         at = {role: f"{prefix}.{name}" for role, name in self.names.items()}
-        specs = [ParamSpec(f"{at[role]}.weight", (rows, self.hidden_size)) for role, rows in self.stored.items()]
-        specs.append(ParamSpec(f"{at['down']}.weight", (self.hidden_size, self.intermediate_size)))
-        specs += [ParamSpec(f"{at[role]}.bias", (rows,)) for role, rows in self.stored.items() if role in self.bias]
+        ws, bs = self.w_suffix, self.b_suffix
+        specs = [ParamSpec(f"{at[role]}{ws}", (rows, self.hidden_size)) for role, rows in self.stored.items()]
+        specs.append(ParamSpec(f"{at['down']}{ws}", (self.hidden_size, self.intermediate_size)))
+        specs += [ParamSpec(f"{at[role]}{bs}", (rows,)) for role, rows in self.stored.items() if role in self.bias]
         if "down" in self.bias:
-            specs.append(ParamSpec(f"{at['down']}.bias", (self.hidden_size,)))
+            specs.append(ParamSpec(f"{at['down']}{bs}", (self.hidden_size,)))
         return specs
 
     def _gate_and_up(self, tensors, at, suffix, roles, device, dtype):
-        """The gate's and the up's tensor named ``suffix`` (``weight`` or ``bias``), each None unless its stored
-        role is among ``roles``."""
+        """The gate's and the up's tensor named by ``suffix`` (the weights' or the biases'), each None unless its
+        stored role is among ``roles``."""
         inter = self.intermediate_size
         if "gate_up" in self.stored:
             if "gate_up" not in roles:
                 return None, None
-            both = tensors[f"{at['gate_up']}.{suffix}"].to(device=device, dtype=dtype)
+            both = tensors[f"{at['gate_up']}{suffix}"].to(device=device, dtype=dtype)
             return both[:inter], both[inter:]
-        return tuple(tensors[f"{at[role]}.{suffix}"].to(device=device, dtype=dtype) if role in roles else None
+        return tuple(tensors[f"{at[role]}{suffix}"].to(device=device, dtype=dtype) if role in roles else None
                      for role in ("gate", "up"))
 
     def bind(self, tensors, prefix, device, dtype) -> None:
         at = {role: f"{prefix}.{name}" for role, name in self.names.items()}
-        gate, up = self._gate_and_up(tensors, at, "weight", self.stored, device, dtype)
+        gate, up = self._gate_and_up(tensors, at, self.w_suffix, self.stored, device, dtype)
         # widths that the activation kernel cannot take in fours keep the gates before the ups
         self.fours = self.intermediate_size % ops.FOURS_WIDTH_MULTIPLE == 0
         join = ops.rows_in_fours if self.fours else (lambda g, u: torch.cat([g, u], dim=0).contiguous())
         self.w_gate_up = decode_weight(join(gate, up), self.tiled_weights)
-        self.w_down = decode_weight(tensors[f"{at['down']}.weight"].to(device=device, dtype=dtype).contiguous(),
+        self.w_down = decode_weight(tensors[f"{at['down']}{self.w_suffix}"].to(device=device, dtype=dtype).contiguous(),
                                     self.tiled_weights)
         if self.bias & set(self.stored):  # laid out as the rows of the joined matrix are; zeros where there is none
             zeros = torch.zeros(self.intermediate_size, dtype=torch.float32, device=device)
             gate_b, up_b = (zeros if b is None else b
-                            for b in self._gate_and_up(tensors, at, "bias", self.bias, device, torch.float32))
+                            for b in self._gate_and_up(tensors, at, self.b_suffix, self.bias, device, torch.float32))
             self.b_gate_up = join(gate_b[:, None], up_b[:, None]).reshape(-1).contiguous()
         if "down" in self.bias:
-            self.b_down = tensors[f"{at['down']}.bias"].to(device=device, dtype=torch.float32).contiguous()
+            self.b_down = tensors[f"{at['down']}{self.b_suffix}"].to(device=device, dtype=torch.float32).contiguous()
 
     def forward(self, x: torch.Tensor, step) -> torch.Tensor:
         act = None
@@ -91,4 +98,15 @@ class GatedMLP(FeedForward):
         return out if self.b_down is None else ops.add_bias(out, self.b_down)
 
 
+class NoFeedForward(FeedForward):
+    """A layer without a feed-forward: ``forward`` returns None and the block adds nothing for it."""
+
+    def __init__(self, spec: PartSpec, *, hidden_size: int):
+        self.hidden_size = int(hidden_size)
+
+    def forward(self, x: torch.Tensor, step):
+        return None
+
+
 FEED_FORWARDS.register("gated_mlp", GatedMLP)
+FEED_FORWARDS.register("none", NoFeedForward)

@@ -4,6 +4,11 @@ eps is added to the mean inside the root; sum, root and product are 32-bit
 (v3/kernels/rmsnorm_inplace_f16.cu:29-62, v3/crates/rvllm-fused/src/reference.rs:58-76).
 ``unit_offset`` selects the zero-centred form of the Gemma checkpoints, where
 the stored weight is the gain minus one.
+
+``rmsnorm_scalar``: the same with one number as the gain of the whole row,
+y = x * rsqrt(mean(x^2) + eps) * g.  Its input may be a residual stream that a
+bf16 model keeps in 32 bits; the output has the activations' type.  ``suffix``
+is what the tensor's name is followed by (``.weight`` if absent).
 """
 
 from __future__ import annotations
@@ -13,7 +18,7 @@ from typing import Optional
 import torch
 
 from ..kernels import ops
-from .base import Norm, ParamSpec
+from .base import Norm, ParamSpec, tensor_path
 from .registry import NORMS
 from .spec import PartSpec
 
@@ -49,4 +54,28 @@ class RMSNorm(Norm):
         return then.forward(residual, out=then_out)
 
 
+class ScalarRMSNorm(Norm):
+    def __init__(self, spec: PartSpec, *, width: int, name: str):
+        self.width = int(width)
+        self.name = name
+        self.eps = float(spec["eps"])
+        self.suffix = str(spec.get("suffix", ".weight"))
+        self.gain: Optional[torch.Tensor] = None
+        self.out_dtype: Optional[torch.dtype] = None
+
+    def param_specs(self, prefix: str) -> list[ParamSpec]:
+        return [ParamSpec(tensor_path(prefix, self.name) + self.suffix, (), init=("normal_about", 1.0, 0.1))]
+
+    def bind(self, tensors, prefix, device, dtype) -> None:
+        self.gain = tensors[tensor_path(prefix, self.name) + self.suffix].to(device).reshape(1).contiguous()
+        self.out_dtype = dtype
+
+    def forward(self, x: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+        return ops.scalar_rmsnorm(x, self.gain, self.eps, self.out_dtype, out=out)
+
+    def forward_rows(self, x: torch.Tensor, rows: torch.Tensor) -> torch.Tensor:
+        return ops.scalar_rmsnorm(x, self.gain, self.eps, self.out_dtype, rows=rows)
+
+
 NORMS.register("rmsnorm", RMSNorm)
+NORMS.register("rmsnorm_scalar", ScalarRMSNorm)

@@ -69,6 +69,9 @@ class ModelSpec:
     head: PartSpec
     prefix: str = "model"
     final_norm_name: str = "norm"  # the final norm's tensor is <prefix>.<final_norm_name>.weight
+    # The residual stream between the layers is 32-bit also where the activations are bf16 (the blocks and norms of
+    # such a model take a 32-bit stream); False: it has the activations' type.
+    residual_float32: bool = False
 
     def __post_init__(self):
         n = len(self.layers)

@@ -33,6 +33,14 @@ def _fill(spec: ParamSpec, seed: int, device, dtype: torch.dtype) -> torch.Tenso
         t = torch.empty(spec.shape, dtype=torch.float32, device=device)
         t.normal_(0.0, float(spec.init[1]), generator=gen)
         return t.to(dtype)
+    if kind == "normal_about":  # (mean, std): gains that are near one
+        t = torch.empty(spec.shape, dtype=torch.float32, device=device)
+        t.normal_(float(spec.init[1]), float(spec.init[2]), generator=gen)
+        return t.to(dtype)
+    if kind == "distinct":  # integer rows whose entries differ, each below init[1]
+        rows, cols = spec.shape
+        picks = torch.rand((rows, int(spec.init[1])), generator=gen, device=device).argsort(dim=1)[:, :cols]
+        return picks.to(torch.int32).contiguous()
     if kind == "randint":
         return torch.randint(int(spec.init[1]), int(spec.init[2]), spec.shape, generator=gen, device=device,
                              dtype=torch.int32)
