@@ -198,7 +198,7 @@ def write_safetensors(path: str | os.PathLike, tensors: dict[str, torch.Tensor],
         if t.dtype not in _NAME_OF:
             raise SafetensorsError(f"cannot store dtype {t.dtype} of {name!r}")
         t = t.detach().cpu().contiguous()
-        raw = t.view(torch.uint8).numpy().tobytes() if t.numel() else b""
+        raw = t.reshape(-1).view(torch.uint8).numpy().tobytes() if t.numel() else b""  # (a single number has no dimension to view)
         header[name] = {"dtype": _NAME_OF[t.dtype], "shape": list(t.shape), "data_offsets": [offset, offset + len(raw)]}
         blobs.append(raw)
         offset += len(raw)
