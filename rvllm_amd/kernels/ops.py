@@ -322,14 +322,35 @@ def gemm_heads(a: torch.Tensor, a_col0: int, w: torch.Tensor, out: Optional[torc
               and gate.shape[0] == m and 0 <= gate_col0 and gate_col0 + heads * n <= gate.shape[1],
               "gemm_heads: the gate must hold the output's columns in its rows")
         gptr, ldg = gate.data_ptr() + gate_col0 * gate.element_size(), gate.stride(0)
+    aptr = a.data_ptr() + a_col0 * a.element_size()
+    if a.dtype == torch.bfloat16 and _mfma_groups_take(aptr, a.stride(0), w, k):
+        _check(library().rv_gemm_groups_mfma(
+            _stream(), aptr, _ptr(w), _ptr(out), None, None, _c_int(heads), _c_int(m), _c_int(n), _c_int(k),
+            _c_ll(a.stride(0)), _c_ll(k), _c_ll(out.stride(0)), _c_ll(k), _c_ll(n * k), _c_ll(n), gptr, _c_ll(ldg),
+            _c_int(0), _c_float(0.0), _c_float(0.0)))
+        return out
     _check(library().rv_gemm_groups_plain(
-        _stream(), a.data_ptr() + a_col0 * a.element_size(), _dt(a), _ptr(w), _dt(w), _ptr(out), _dt(out), None, None,
+        _stream(), aptr, _dt(a), _ptr(w), _dt(w), _ptr(out), _dt(out), None, None,
         _c_int(heads), _c_int(m), _c_int(n), _c_int(k), _c_ll(a.stride(0)), _c_ll(k), _c_ll(out.stride(0)), _c_ll(k),
         _c_ll(n * k), _c_ll(n), gptr, _c_ll(ldg)))
     return out
 
 
-MOE_TILE_ROWS = 64  # rows of one expert that a block of the grouped product takes
+def _mfma_groups_take(aptr: int, lda: int, w: torch.Tensor, k: int) -> bool:
+    """Whether the matrix-core kernel for products by group reads these operands: 16 bytes a lane at a time."""
+    return k % 8 == 0 and lda % 8 == 0 and aptr % 16 == 0 and w.data_ptr() % 16 == 0
+
+
+MOE_TILE_ROWS = 64  # rows of one expert that a block of the 32-bit grouped product takes
+MOE_TILE_ROWS_MFMA = 16  # and a wave of the matrix-core one
+
+
+def moe_tile_rows(dtype: torch.dtype, *inner_sizes: int) -> int:
+    """The rows a tile of the sorted order holds for products of this type whose summed sizes are
+    ``inner_sizes``: 16 where the matrix-core kernel takes them (bf16, sizes that are multiples of 8), else 64."""
+    if dtype == torch.bfloat16 and all(k % 8 == 0 for k in inner_sizes):
+        return MOE_TILE_ROWS_MFMA
+    return MOE_TILE_ROWS
 
 
 def moe_capacity(num_tokens: int, top: int, experts: int, tile: int = MOE_TILE_ROWS) -> int:
@@ -357,24 +378,40 @@ def moe_route(token_ids: torch.Tensor, num_tokens: int, table: torch.Tensor, exp
 
 
 def gemm_experts(a: torch.Tensor, w: torch.Tensor, tile_group: torch.Tensor, row_index: Optional[torch.Tensor] = None,
-                 out: Optional[torch.Tensor] = None) -> torch.Tensor:
+                 out: Optional[torch.Tensor] = None, tile: int = MOE_TILE_ROWS,
+                 glu: Optional[tuple[float, float]] = None) -> torch.Tensor:
     """``out[r] = a[row_index[r]] @ w[tile_group[r // tile]]^T`` for the sorted rows of ``moe_route``; ``w`` is
     ``[experts, N, K]``.  Without ``row_index`` the rows of ``a`` are the sorted rows themselves.  Rows of tiles
-    without an expert are left as they are."""
+    without an expert are left as they are.  ``tile`` is the route's (``moe_tile_rows``): 16 runs the matrix-core
+    kernel, 64 the 32-bit one.  ``glu`` = (limit, alpha), with tiles of 16 only: ``w`` holds each expert's gate rows
+    and then its up rows, and the result is the clamped gated activation of the two products, ``[rows, N / 2]``."""
     _gpu(a, w, tile_group, row_index, out)
     _i32(tile_group)
     _need(a.dim() == 2 and w.dim() == 3 and a.dtype == w.dtype and a.dtype in _DT and a.shape[1] == w.shape[2],
           "gemm_experts: rows [*, K] against matrices [experts, N, K] of one type expected")
-    m = tile_group.numel() * MOE_TILE_ROWS
+    _need(tile in (MOE_TILE_ROWS, MOE_TILE_ROWS_MFMA), f"gemm_experts: tiles of {tile} rows")
+    m = tile_group.numel() * tile
     if row_index is not None:
         _i32(row_index)
         _need(row_index.numel() == m, "gemm_experts: one source row for every sorted row")
     else:
         _need(a.shape[0] == m, "gemm_experts: the rows must be the sorted rows")
     _, n, k = w.shape
+    if glu is not None:
+        _need(n % 2 == 0 and tile == MOE_TILE_ROWS_MFMA, "gemm_experts: the activation is applied by the matrix-core kernel")
+        n //= 2
     if out is None:
         out = torch.empty((m, n), dtype=a.dtype, device=a.device)
     _need(out.shape == (m, n) and out.dtype == a.dtype, "gemm_experts: bad out")
+    if tile == MOE_TILE_ROWS_MFMA:
+        _need(a.dtype == torch.bfloat16 and _mfma_groups_take(a.data_ptr(), a.stride(0), w, k),
+              "gemm_experts: tiles of 16 rows are the matrix-core kernel's: bf16, sizes that are multiples of 8")
+        limit, alpha = glu if glu is not None else (0.0, 0.0)
+        _check(library().rv_gemm_groups_mfma(
+            _stream(), _ptr(a), _ptr(w), _ptr(out), _ptr(row_index), _ptr(tile_group), _c_int(0), _c_int(m), _c_int(n),
+            _c_int(k), _c_ll(a.stride(0)), _c_ll(k), _c_ll(n), _c_ll(0), _c_ll(w.shape[1] * k), _c_ll(0), None, _c_ll(0),
+            _c_int(int(glu is not None)), _c_float(limit), _c_float(alpha)))
+        return out
     _check(library().rv_gemm_groups_plain(
         _stream(), _ptr(a), _dt(a), _ptr(w), _dt(w), _ptr(out), _dt(out), _ptr(row_index), _ptr(tile_group), _c_int(0),
         _c_int(m), _c_int(n), _c_int(k), _c_ll(a.stride(0)), _c_ll(k), _c_ll(n), _c_ll(0), _c_ll(n * k), _c_ll(0),

@@ -200,7 +200,8 @@ def test_the_compressed_vector_is_normed_and_written_for_both_products(dtype, ra
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("rows,heads,n,k", [(1, 6, 96, 64), (70, 3, 24, 40), (130, 17, 10, 7), (9, 1, 128, 128)])
+@pytest.mark.parametrize("rows,heads,n,k", [(1, 6, 96, 64), (70, 3, 24, 40), (130, 17, 10, 7), (9, 1, 128, 128),
+                                            (16, 2, 17, 72), (300, 5, 250, 16), (33, 8, 66, 200)])
 def test_products_by_head_with_and_without_a_gate(dtype, rows, heads, n, k):
     g = torch.Generator().manual_seed(rows)
     lead = 16
@@ -215,7 +216,8 @@ def test_products_by_head_with_and_without_a_gate(dtype, rows, heads, n, k):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("tokens,experts,top,width,inner", [(1, 8, 1, 64, 24), (7, 5, 2, 40, 20), (300, 70, 3, 96, 36),
-                                                           (65, 3, 3, 100, 50), (130, 2, 1, 72, 8)])
+                                                           (65, 3, 3, 100, 50), (130, 2, 1, 72, 8), (33, 4, 2, 256, 200),
+                                                           (16, 1, 1, 32, 72), (17, 9, 4, 128, 64)])
 def test_experts_chosen_by_the_tokens_id(dtype, tokens, experts, top, width, inner):
     g = torch.Generator().manual_seed(tokens + experts)
     vocab, limit = 53, 0.8
@@ -231,17 +233,26 @@ def test_experts_chosen_by_the_tokens_id(dtype, tokens, experts, top, width, inn
     want = PP.routed_ff(h.double(), ids.tolist(), {k: (v.double() if v.is_floating_point() else v) for k, v in w.items()}, "", mlp)
     w_gu = dev(torch.stack([torch.cat([w[f"e{e}.gate"], w[f"e{e}.up"]]) for e in range(experts)]))
     w_down = dev(torch.stack([w[f"e{e}.down"] for e in range(experts)]))
-    slot_of, row_token, tile_group = ops.moe_route(dev(ids), tokens, dev(table), experts)
+    tile = ops.moe_tile_rows(dtype, width, inner)  # 16 rows and the matrix cores for bf16 sizes in eights, else 64
+    assert tile == (16 if dtype == torch.bfloat16 and width % 8 == 0 and inner % 8 == 0 else 64)
+    slot_of, row_token, tile_group = ops.moe_route(dev(ids), tokens, dev(table), experts, tile)
     # the sorted order: every choice has a row of its own in a tile of its expert, rows know their tokens
     so, rt, tg = slot_of.cpu().view(tokens, top), row_token.cpu(), tile_group.cpu()
     assert so.min() >= 0 and so.flatten().unique().numel() == tokens * top
     for t in range(tokens):
         for c in range(top):
-            assert rt[so[t, c]] == t and tg[so[t, c] // ops.MOE_TILE_ROWS] == table[ids[t], c]
+            assert rt[so[t, c]] == t and tg[so[t, c] // tile] == table[ids[t], c]
     assert int((rt >= 0).sum()) == tokens * top
-    act = ops.clamped_glu(ops.gemm_experts(dev(h), w_gu, tile_group, row_index=row_token), limit, 1.702)
-    got = ops.moe_combine(ops.gemm_experts(act, w_down, tile_group), slot_of, top, 1.0 / top, tokens)
+    if tile == 16:  # the activation inside the product
+        act = ops.gemm_experts(dev(h), w_gu, tile_group, row_index=row_token, tile=tile, glu=(limit, 1.702))
+    else:
+        act = ops.clamped_glu(ops.gemm_experts(dev(h), w_gu, tile_group, row_index=row_token, tile=tile), limit, 1.702)
+    got = ops.moe_combine(ops.gemm_experts(act, w_down, tile_group, tile=tile), slot_of, top, 1.0 / top, tokens)
     close(got, want, dtype)
+    if tile == 16:  # the same through the kernels that take any size
+        s64, r64, t64 = ops.moe_route(dev(ids), tokens, dev(table), experts, 64)
+        act = ops.clamped_glu(ops.gemm_experts(dev(h), w_gu, t64, row_index=r64), limit, 1.702)
+        close(ops.moe_combine(ops.gemm_experts(act, w_down, t64), s64, top, 1.0 / top, tokens), want, dtype, "tiles of 64")
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
