@@ -3,6 +3,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--context 8192] [--layers L]
     python bench.py --workload 12b|27b [--requests N] [--layers L]     (another measurement, see WORKLOADS)
+    python bench.py --design pinorax [--size s|l] [--layers L]          (another measurement, see DESIGN_SIZES)
 
 Default run: the layer sizes of the 4B-sized configuration (34 layers, 5
 sliding : 1 global, hidden 2560, 8 query / 4 key-value heads of 256, GeGLU
@@ -319,6 +320,93 @@ def run_workload(name: str, requests, layers) -> int:
     return 0
 
 
+# ---- another design beside the dense decoder, layer for layer ------------------------------------------------
+# Sizes that resemble a real model's layers.  The Pinorax layers: latent attention (``heads`` of ``dim`` / ``vdim``
+# over a compressed vector of ``kv_rank``), the first layer with a dense feed-forward, the others with experts
+# chosen by token id and a shared expert.  Beside it the dense decoder at equal size: the same width, layers,
+# vocabulary and heads, a feed-forward as wide as what a Pinorax token uses (top * expert + shared).
+DESIGN_SIZES = {
+    "s": dict(width=2048, heads=16, dim=128, vdim=128, kv_rank=256, dense_ff=8192, experts=32, top=2, expert_ff=1024,
+              shared_ff=2048, vocab=32000, kv_heads=4),
+    "l": dict(width=4096, heads=32, dim=128, vdim=128, kv_rank=256, dense_ff=12288, experts=64, top=4, expert_ff=1024,
+              shared_ff=2048, vocab=32000, kv_heads=8),
+}
+
+
+def design_configs(size: dict, layers: int, positions: int):
+    from rvllm_amd.config.gemma3 import Gemma3Config
+    from rvllm_amd.config.pinorax import PinoraxConfig
+
+    mixer = {"heads": size["heads"], "dim": size["dim"], "vdim": size["vdim"], "kv_rank": size["kv_rank"],
+             "scale": size["dim"] ** -0.5}
+    moe = {"kind": "moe", "expert": {"ff": size["expert_ff"], "limit": 7.0},
+           "router": {"experts": size["experts"], "top": size["top"]}, "shared": {"ff": size["shared_ff"], "limit": 7.0}}
+    pinorax = PinoraxConfig.from_dict({
+        "architecture": "Pinorax", "vocab": size["vocab"], "width": size["width"], "max_positions": positions,
+        "norm": {"eps": 1e-6}, "residual_mult": 0.5, "logit_softcap": 30.0,
+        "layers": [{"type": "latent_attention", "mixer": mixer,
+                    "mlp": {"kind": "dense", "ff": size["dense_ff"]} if i == 0 else moe} for i in range(layers)],
+    }, "bench configuration")
+    used_ff = size["top"] * size["expert_ff"] + size["shared_ff"]
+    dense = Gemma3Config.from_dict(dict(
+        GEMMA3_4B, num_hidden_layers=layers, hidden_size=size["width"], num_attention_heads=size["heads"],
+        num_key_value_heads=size["kv_heads"], head_dim=size["dim"], intermediate_size=used_ff, vocab_size=size["vocab"],
+        query_pre_attn_scalar=size["dim"], max_position_embeddings=positions, sliding_window_pattern=1),
+        "bench configuration")  # every layer global: all keys visible, as in Pinorax's layers
+    return pinorax, dense
+
+
+def run_design(args) -> int:
+    """Prefill and decode of the Pinorax design beside the dense decoder at equal size; one JSON line."""
+    import torch
+
+    from rvllm_amd.config.engine_config import EngineConfig
+    from rvllm_amd.engine.runner import ModelRunner
+    from rvllm_amd.sampling.params import SamplingParams
+    from rvllm_amd.sampling.sampler import Sampler, SplitMix64
+    import rvllm_amd.models  # noqa: F401
+
+    size = DESIGN_SIZES[args.size]
+    layers = args.layers if args.layers != FULL_LAYERS else 8
+    context, T = args.context, args.prefill_tokens
+    batches = [b for b in (8, 64) if not (args.no_points and b != 8)]
+    steps_total = args.steps + args.warmup + 8
+    positions = max(context + steps_total + 16, T)
+    out = {"metric": f"prefill and decode of Pinorax beside the dense decoder, size {args.size}", "unit": "ms",
+           "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic: random weights, caches filled "
+           "with random values, uniform token ids", "config": dict(size, layers=layers, context=context, prefill_tokens=T),
+           "designs": {}}
+    for name, cfg in zip(("pinorax", "dense"), design_configs(size, layers, positions)):
+        engine_cfg = EngineConfig(dtype=args.dtype, page_size=args.page_size, max_model_len=positions,
+                                  max_num_seqs=max(batches), max_num_batched_tokens=max(T, max(batches)),
+                                  max_prefill_chunk=T, max_cache_tokens=max(batches) * (context + steps_total + 16),
+                                  use_graphs=bool(args.graphs))
+        log(f"{name}: building {layers} layers with random weights")
+        runner = ModelRunner.from_random(cfg, 0, engine_cfg)
+        torch.cuda.synchronize()
+        parts = (torch, runner, Sampler(size["vocab"]), SamplingParams, SplitMix64)
+        numbers = {"weights_GiB": round(runner.weight_bytes / 2**30, 2), "cache_GiB": round(runner.storage.bytes / 2**30, 2)}
+        for b in batches:
+            sec = time_decode(parts, b, context, args.steps, args.warmup)
+            numbers[f"decode_b{b}_ms"] = round(sec * 1e3, 4)
+            numbers[f"decode_b{b}_tok_s"] = round(b / sec, 1)
+            log(f"{name}: decode batch {b} at context {context}: {sec * 1e3:.3f} ms/step")
+        if not args.no_prefill:
+            psec, pmin = time_prefill(parts, T, repeats=5)
+            numbers["prefill_ms"] = round(psec * 1e3, 3)
+            numbers["prefill_tok_s"] = round(T / psec, 1)
+            log(f"{name}: prefill {T} tokens: {psec * 1e3:.2f} ms")
+        out["designs"][name] = numbers
+        del runner, parts
+        import gc
+        gc.collect()
+        torch.cuda.empty_cache()
+    p, d = out["designs"]["pinorax"], out["designs"]["dense"]
+    out["pinorax_over_dense"] = {k: round(p[k] / d[k], 3) for k in p if k.endswith("_ms") and k in d}
+    print(json.dumps(out), flush=True)
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -343,10 +431,17 @@ def main() -> int:
     ap.add_argument("--workload", choices=sorted(WORKLOADS), help="instead of the default run: an engine workload of a "
                     "larger configuration (requests through the scheduler); --requests and --layers shrink it")
     ap.add_argument("--requests", type=int, default=0)
+    ap.add_argument("--design", choices=["pinorax"], help="instead of the default run: prefill and decode of another "
+                    "design of the framework beside the dense decoder at equal size (--size, --layers, --context)")
+    ap.add_argument("--size", choices=sorted(DESIGN_SIZES), default="s")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this single-GPU engine", flush=True)
         return 2
+    if args.design:
+        if args.context == 8192:
+            args.context = 4096
+        return run_design(args)
     if args.workload:
         return run_workload(args.workload, args.requests, args.layers if args.layers != FULL_LAYERS else 0)
 

@@ -111,7 +111,7 @@ extern "C" int rv_gemm_groups_plain(hipStream_t stream, const void* a, int a_dty
 // The same products in bf16 on the matrix cores (MFMA 16x16x32), for both forms.  The product is taken
 // transposed, C^T = W A^T, as in the few-row product: 16 rows of W are the A operand and 16 rows of a (tokens) the
 // B operand, both read straight from memory in the order the instruction sums them (8 consecutive k a lane, 16
-// bytes), so a lane ends up with 4 consecutive outputs of one token.  A wave takes 16 tokens against NT tiles of
+// bytes), so a lane ends up with 4 consecutive outputs of one token.  A wave takes 16 tokens against 1 or 4 tiles of
 // 16 rows of W (the tokens' values are read once for all of them); the four waves of a block take neighbouring
 // rows of W.  Tiles of rows are 16 here (tile_group has an entry for every 16 rows).  Sums are 32-bit.
 //
@@ -140,16 +140,19 @@ struct GroupsParams {
   int vec_store;
 };
 
-#define GG_NT 4
-
-template <bool GLU>
+// NT tiles of 16 rows of W a wave: 4 where many tokens share them (a prompt), 1 where the tokens are few and the
+// launch needs every wave it can get to draw the memory's rate (decoding).  The loop over k is written out UNROLL
+// steps at a time with every read of the steps asked for before the first product, so that a wave has a dozen
+// 16-byte reads in flight.
+template <int NT, bool GLU>
 __global__ void __launch_bounds__(256) gemm_groups_mfma_kernel(const GroupsParams P) {
+  constexpr int UNROLL = NT * (GLU ? 2 : 1) >= 4 ? 2 : 4;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r16 = lane & 15, kb = lane >> 4;
   const int group = P.tile_group ? P.tile_group[blockIdx.y] : (int)blockIdx.z;
   if (group < 0) return;  // the whole block alike
   const int m0 = blockIdx.y * 16;
-  const int n0 = (blockIdx.x * 4 + wave) * 16 * GG_NT;
+  const int n0 = (blockIdx.x * 4 + wave) * 16 * NT;
   if (n0 >= P.N) return;  // the whole wave
   const uint16_t* a = P.a + (size_t)group * P.a_group_stride;
   const uint16_t* w = P.w + (size_t)group * P.w_group_stride;
@@ -157,43 +160,48 @@ __global__ void __launch_bounds__(256) gemm_groups_mfma_kernel(const GroupsParam
   long long a_row = -1;
   if (am < P.M) a_row = P.row_index ? P.row_index[am] : am;
   const uint16_t* xr = a + (size_t)(a_row >= 0 ? a_row : 0) * P.lda;
-  const uint16_t* wr[GG_NT];
+  const uint16_t* wr[NT];
 #pragma unroll
-  for (int t = 0; t < GG_NT; ++t) {
+  for (int t = 0; t < NT; ++t) {
     int n = n0 + t * 16 + r16;
     n = n < P.N ? n : P.N - 1;  // rows past the end repeat the last one and are not stored
     wr[t] = w + (size_t)n * P.ldw;
   }
   const size_t up_rows = (size_t)P.N * P.ldw;  // GLU: the up rows follow the N gate rows
-  gg_f32x4 acc[GG_NT], acc_up[GG_NT];
+  gg_f32x4 acc[NT], acc_up[NT];
 #pragma unroll
-  for (int t = 0; t < GG_NT; ++t) {
+  for (int t = 0; t < NT; ++t) {
     acc[t] = (gg_f32x4){0.f, 0.f, 0.f, 0.f};
     acc_up[t] = (gg_f32x4){0.f, 0.f, 0.f, 0.f};
   }
-  for (int k0 = 0; k0 < P.K; k0 += 32) {
-    const int k = k0 + kb * 8;
-    const bool in = k < P.K;
-    const int kk = in ? k : 0;  // reads are unconditional, from an address that exists; what lies past K is zeroed
-    GgFrag8 xf, wf[GG_NT], uf[GG_NT];
-    xf.u4 = *(const uint4*)(xr + kk);
+  for (int k0 = 0; k0 < P.K; k0 += 32 * UNROLL) {
+    GgFrag8 xf[UNROLL], wf[UNROLL][NT], uf[UNROLL][NT];
 #pragma unroll
-    for (int t = 0; t < GG_NT; ++t) {
-      wf[t].u4 = *(const uint4*)(wr[t] + kk);
-      if constexpr (GLU) uf[t].u4 = *(const uint4*)(wr[t] + up_rows + kk);
+    for (int u = 0; u < UNROLL; ++u) {
+      const int k = k0 + u * 32 + kb * 8;
+      const int kk = k < P.K ? k : 0;  // reads are unconditional, from an address that exists; what lies past K is zeroed
+      xf[u].u4 = *(const uint4*)(xr + kk);
+#pragma unroll
+      for (int t = 0; t < NT; ++t) {
+        wf[u][t].u4 = *(const uint4*)(wr[t] + kk);
+        if constexpr (GLU) uf[u][t].u4 = *(const uint4*)(wr[t] + up_rows + kk);
+      }
     }
-    if (!in || a_row < 0) xf.u4 = make_uint4(0, 0, 0, 0);
 #pragma unroll
-    for (int t = 0; t < GG_NT; ++t) {
-      acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[t].v, xf.v, acc[t], 0, 0, 0);
-      if constexpr (GLU) acc_up[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(uf[t].v, xf.v, acc_up[t], 0, 0, 0);
+    for (int u = 0; u < UNROLL; ++u) {
+      if (k0 + u * 32 + kb * 8 >= P.K || a_row < 0) xf[u].u4 = make_uint4(0, 0, 0, 0);
+#pragma unroll
+      for (int t = 0; t < NT; ++t) {
+        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[u][t].v, xf[u].v, acc[t], 0, 0, 0);
+        if constexpr (GLU) acc_up[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(uf[u][t].v, xf[u].v, acc_up[t], 0, 0, 0);
+      }
     }
   }
   if (am >= P.M) return;
   uint16_t* cr = P.c + (size_t)group * P.c_group_stride + (size_t)am * P.ldc;
   const uint16_t* gr = P.gate ? P.gate + (size_t)group * P.c_group_stride + (size_t)am * P.ldg : nullptr;
 #pragma unroll
-  for (int t = 0; t < GG_NT; ++t) {
+  for (int t = 0; t < NT; ++t) {
     const int n = n0 + t * 16 + kb * 4;
     float v[4];
 #pragma unroll
@@ -229,7 +237,7 @@ extern "C" int rv_gemm_groups_mfma(hipStream_t stream, const void* a, const void
                                    const int* tile_group, int groups, int M, int N, int K, long long lda,
                                    long long ldw, long long ldc, long long a_group_stride, long long w_group_stride,
                                    long long c_group_stride, const void* gate, long long ldg, int glu, float limit,
-                                   float alpha) {
+                                   float alpha, int tiles_a_wave) {
   RV_CHECK(M >= 0 && N > 0 && K > 0 && groups >= 0, "gemm_groups_mfma: bad sizes M=%d N=%d K=%d groups=%d", M, N, K, groups);
   RV_CHECK((groups > 0) == (tile_group == nullptr), "gemm_groups_mfma: either a number of groups or the groups of the row tiles");
   RV_CHECK(K % 8 == 0 && lda % 8 == 0 && ldw % 8 == 0 && a_group_stride % 8 == 0 && w_group_stride % 8 == 0 &&
@@ -238,6 +246,7 @@ extern "C" int rv_gemm_groups_mfma(hipStream_t stream, const void* a, const void
            "16-byte aligned");
   RV_CHECK(lda >= K && ldw >= K && ldc >= N && (gate == nullptr || ldg >= N), "gemm_groups_mfma: rows too short");
   RV_CHECK(!glu || (gate == nullptr && limit > 0.f), "gemm_groups_mfma: the gated activation takes a limit and no gate");
+  RV_CHECK(tiles_a_wave == 1 || tiles_a_wave == 4, "gemm_groups_mfma: 1 or 4 tiles of rows a wave, not %d", tiles_a_wave);
   if (M == 0) return 0;
   GroupsParams P;
   P.a = (const uint16_t*)a;
@@ -251,10 +260,12 @@ extern "C" int rv_gemm_groups_mfma(hipStream_t stream, const void* a, const void
   P.a_group_stride = a_group_stride, P.w_group_stride = w_group_stride, P.c_group_stride = c_group_stride;
   P.limit = limit, P.alpha = alpha;
   P.vec_store = (ldc % 4 == 0 && c_group_stride % 4 == 0 && ((uintptr_t)c & 7) == 0) ? 1 : 0;
-  dim3 grid(rv_div_up(N, 16 * GG_NT * 4), rv_div_up(M, 16), groups > 0 ? groups : 1), block(256);
+  dim3 grid(rv_div_up(N, 16 * tiles_a_wave * 4), rv_div_up(M, 16), groups > 0 ? groups : 1), block(256);
   RV_CHECK(grid.y < 65536 && grid.z < 65536, "gemm_groups_mfma: too many row tiles or groups for one launch");
-  if (glu) gemm_groups_mfma_kernel<true><<<grid, block, 0, stream>>>(P);
-  else gemm_groups_mfma_kernel<false><<<grid, block, 0, stream>>>(P);
+  if (glu && tiles_a_wave == 1) gemm_groups_mfma_kernel<1, true><<<grid, block, 0, stream>>>(P);
+  else if (glu) gemm_groups_mfma_kernel<4, true><<<grid, block, 0, stream>>>(P);
+  else if (tiles_a_wave == 1) gemm_groups_mfma_kernel<1, false><<<grid, block, 0, stream>>>(P);
+  else gemm_groups_mfma_kernel<4, false><<<grid, block, 0, stream>>>(P);
   RV_LAUNCH_CHECK("gemm_groups_mfma");
   return 0;
 }

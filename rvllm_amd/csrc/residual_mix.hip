@@ -48,17 +48,55 @@ extern "C" int rv_scalar_rmsnorm(hipStream_t stream, const void* x, int x_dtype,
   return 0;
 }
 
-// A branch's value: stored as T, or the sum of `slices` 32-bit partial sums added in their order.
-template <typename T>
-__device__ __forceinline__ float rm_branch(const void* p, int slices, long long stride, size_t at) {
-  if (p == nullptr) return 0.f;
-  if (slices == 0) return rv_to_float(((const T*)p)[at]);
-  float v = 0.f;
-  for (int s = 0; s < slices; ++s) v += ((const float*)p)[(size_t)s * stride + at];
-  return v;
+// V consecutive values of a branch (V is 1 or 4): stored as T, or the sum of `slices` 32-bit partial sums.
+template <typename T, int V>
+__device__ __forceinline__ void rm_branch_vec(const void* p, int slices, long long stride, size_t at, float* out) {
+#pragma unroll
+  for (int v = 0; v < V; ++v) out[v] = 0.f;
+  if (p == nullptr) return;
+  if (slices == 0) {
+    if constexpr (V == 4 && sizeof(T) == 2) {
+      const uint2 q = *(const uint2*)((const uint16_t*)p + at);
+      out[0] = __uint_as_float(q.x << 16), out[1] = __uint_as_float(q.x & 0xffff0000u);
+      out[2] = __uint_as_float(q.y << 16), out[3] = __uint_as_float(q.y & 0xffff0000u);
+    } else if constexpr (V == 4) {
+      const float4 q = *(const float4*)((const float*)p + at);
+      out[0] = q.x, out[1] = q.y, out[2] = q.z, out[3] = q.w;
+    } else {
+      out[0] = rv_to_float(((const T*)p)[at]);
+    }
+    return;
+  }
+  for (int s = 0; s < slices; ++s) {
+    const float* q = (const float*)p + (size_t)s * stride + at;
+    if constexpr (V == 4) {
+      const float4 r = *(const float4*)q;
+      out[0] += r.x, out[1] += r.y, out[2] += r.z, out[3] += r.w;
+    } else {
+      out[0] += q[0];
+    }
+  }
 }
 
-template <typename T>
+template <int V>
+__device__ __forceinline__ void rm_load(const float* p, float* out) {
+  if constexpr (V == 4) {
+    const float4 q = *(const float4*)p;
+    out[0] = q.x, out[1] = q.y, out[2] = q.z, out[3] = q.w;
+  } else {
+    out[0] = p[0];
+  }
+}
+template <int V>
+__device__ __forceinline__ void rm_store(float* p, const float* in) {
+  if constexpr (V == 4) *(float4*)p = make_float4(in[0], in[1], in[2], in[3]);
+  else p[0] = in[0];
+}
+
+// V values a thread and turn: 4 where the width is a multiple of 4 (16-byte reads of the streams), else 1.  Every
+// stream of the history is read before anything is written, so that the reads are on their way together.
+#define RM_MAX_TERMS_AT_ONCE 8
+template <typename T, int V>
 __global__ void __launch_bounds__(RM_THREADS)
 residual_mix_kernel(float* __restrict__ x, const void* __restrict__ a, int a_slices, long long a_stride,
                     const void* __restrict__ f, int f_slices, long long f_stride, float mult,
@@ -68,31 +106,54 @@ residual_mix_kernel(float* __restrict__ x, const void* __restrict__ a, int a_sli
   __shared__ float scratch[16];
   const size_t row0 = (size_t)blockIdx.x * width;
   float ss = 0.f;
-  for (int i = threadIdx.x; i < width; i += RM_THREADS) {
+  for (int i = threadIdx.x * V; i < width; i += RM_THREADS * V) {
     const size_t at = row0 + i;
-    const float x_in = x[at];
-    const float branch = rm_branch<T>(a, a_slices, a_stride, at) + rm_branch<T>(f, f_slices, f_stride, at);
-    const float x_new = fmaf(mult, branch, x_in);
-    float out = x_new;
+    float x_in[V], br_a[V], br_f[V], x_new[V], out[V];
+    rm_load<V>(x + at, x_in);
+    rm_branch_vec<T, V>(a, a_slices, a_stride, at, br_a);
+    rm_branch_vec<T, V>(f, f_slices, f_stride, at, br_f);
+#pragma unroll
+    for (int v = 0; v < V; ++v) out[v] = x_new[v] = fmaf(mult, br_a[v] + br_f[v], x_in[v]);
     if (history != nullptr) {
-      if (seed_history) history[at] = x_in;  // the first layer's input is the embedding's output, X_0
-      history[(size_t)(terms - 1) * history_stride + at] = x_new;
-      out = 0.f;
-      for (int j = 0; j + 1 < terms; ++j) {
-        const float xj = (j == 0 && seed_history) ? x_in : history[(size_t)j * history_stride + at];
-        out = fmaf(rv_load_w(depth_w, depth_w_f32, j), xj, out);
+#pragma unroll
+      for (int v = 0; v < V; ++v) out[v] = 0.f;
+      for (int j0 = 0; j0 + 1 < terms; j0 += RM_MAX_TERMS_AT_ONCE) {
+        float xj[RM_MAX_TERMS_AT_ONCE][V];
+#pragma unroll
+        for (int jj = 0; jj < RM_MAX_TERMS_AT_ONCE; ++jj) {  // a stream past the last repeats it and weighs nothing
+          const int j = j0 + jj + 1 < terms ? j0 + jj : terms - 2;
+          rm_load<V>(((j == 0 && seed_history) ? x : history + (size_t)j * history_stride) + at, xj[jj]);
+        }
+#pragma unroll
+        for (int jj = 0; jj < RM_MAX_TERMS_AT_ONCE; ++jj) {
+          if (j0 + jj + 1 < terms) {
+            const float wj = rv_load_w(depth_w, depth_w_f32, j0 + jj);
+#pragma unroll
+            for (int v = 0; v < V; ++v) out[v] = fmaf(wj, xj[jj][v], out[v]);
+          }
+        }
       }
-      out = fmaf(rv_load_w(depth_w, depth_w_f32, terms - 1), x_new, out);
+      const float w_last = rv_load_w(depth_w, depth_w_f32, terms - 1);
+#pragma unroll
+      for (int v = 0; v < V; ++v) out[v] = fmaf(w_last, x_new[v], out[v]);
+      if (seed_history) rm_store<V>(history + at, x_in);  // the first layer's input is the embedding's output, X_0
+      rm_store<V>(history + (size_t)(terms - 1) * history_stride + at, x_new);
     }
-    x[at] = out;
-    ss = fmaf(out, out, ss);
+    rm_store<V>(x + at, out);
+#pragma unroll
+    for (int v = 0; v < V; ++v) ss = fmaf(out[v], out[v], ss);
   }
   if (next == nullptr) return;
   ss = rv_block_sum(ss, scratch);
   const float inv = 1.0f / sqrtf(ss / (float)width + eps_next);
   const float gain = rv_load_w(g_next, g_next_f32, 0);
   // every thread reads back what it wrote itself
-  for (int i = threadIdx.x; i < width; i += RM_THREADS) next[row0 + i] = rv_from_float<T>(x[row0 + i] * inv * gain);
+  for (int i = threadIdx.x * V; i < width; i += RM_THREADS * V) {
+    float o[V];
+    rm_load<V>(x + row0 + i, o);
+#pragma unroll
+    for (int v = 0; v < V; ++v) next[row0 + i + v] = rv_from_float<T>(o[v] * inv * gain);
+  }
 }
 
 // x [rows, width] float, in place.  a, f: branches of type `dtype` [rows, width] (slices 0) or 32-bit partial sums
@@ -112,12 +173,15 @@ extern "C" int rv_residual_mix(hipStream_t stream, float* x, const void* a, int 
   RV_CHECK((g_next == nullptr) == (next == nullptr), "residual_mix: the next norm needs both gain and output");
   if (rows == 0) return 0;
   dim3 grid(rows), block(RM_THREADS);
-#define RV_RM(T)                                                                                                    \
-  residual_mix_kernel<T><<<grid, block, 0, stream>>>(x, a, a_slices, a_stride, f, f_slices, f_stride, mult, history, \
-                                                     history_stride, terms, seed_history, depth_w, depth_w_f32,     \
-                                                     g_next, g_next_f32, (T*)next, eps_next, width)
-  if (dtype == RV_F32) RV_RM(float);
-  else if (dtype == RV_BF16) RV_RM(bf16_t);
+  // four values a thread where rows, streams and partial sums all start on 16-byte boundaries
+  const bool vec = width % 4 == 0 && history_stride % 4 == 0 && a_stride % 4 == 0 && f_stride % 4 == 0 &&
+                   (((uintptr_t)x | (uintptr_t)a | (uintptr_t)f | (uintptr_t)history) & 15) == 0;
+#define RV_RM(T, V)                                                                                                    \
+  residual_mix_kernel<T, V><<<grid, block, 0, stream>>>(x, a, a_slices, a_stride, f, f_slices, f_stride, mult, history, \
+                                                        history_stride, terms, seed_history, depth_w, depth_w_f32,     \
+                                                        g_next, g_next_f32, (T*)next, eps_next, width)
+  if (dtype == RV_F32) { if (vec) RV_RM(float, 4); else RV_RM(float, 1); }
+  else if (dtype == RV_BF16) { if (vec) RV_RM(bf16_t, 4); else RV_RM(bf16_t, 1); }
   else return rv_fail("residual_mix: unsupported dtype %d", dtype);
 #undef RV_RM
   RV_LAUNCH_CHECK("residual_mix");

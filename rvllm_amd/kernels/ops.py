@@ -327,13 +327,18 @@ def gemm_heads(a: torch.Tensor, a_col0: int, w: torch.Tensor, out: Optional[torc
         _check(library().rv_gemm_groups_mfma(
             _stream(), aptr, _ptr(w), _ptr(out), None, None, _c_int(heads), _c_int(m), _c_int(n), _c_int(k),
             _c_ll(a.stride(0)), _c_ll(k), _c_ll(out.stride(0)), _c_ll(k), _c_ll(n * k), _c_ll(n), gptr, _c_ll(ldg),
-            _c_int(0), _c_float(0.0), _c_float(0.0)))
+            _c_int(0), _c_float(0.0), _c_float(0.0), _c_int(1 if m <= MFMA_GROUPS_FEW_ROWS else 4)))
         return out
     _check(library().rv_gemm_groups_plain(
         _stream(), aptr, _dt(a), _ptr(w), _dt(w), _ptr(out), _dt(out), None, None,
         _c_int(heads), _c_int(m), _c_int(n), _c_int(k), _c_ll(a.stride(0)), _c_ll(k), _c_ll(out.stride(0)), _c_ll(k),
         _c_ll(n * k), _c_ll(n), gptr, _c_ll(ldg)))
     return out
+
+
+# Up to this many rows a wave of the matrix-core kernel for products by group takes one tile of 16 rows of the
+# matrix, so that a launch has waves enough to draw the memory's rate; beyond, four, which share the rows' values.
+MFMA_GROUPS_FEW_ROWS = 256
 
 
 def _mfma_groups_take(aptr: int, lda: int, w: torch.Tensor, k: int) -> bool:
@@ -410,7 +415,8 @@ def gemm_experts(a: torch.Tensor, w: torch.Tensor, tile_group: torch.Tensor, row
         _check(library().rv_gemm_groups_mfma(
             _stream(), _ptr(a), _ptr(w), _ptr(out), _ptr(row_index), _ptr(tile_group), _c_int(0), _c_int(m), _c_int(n),
             _c_int(k), _c_ll(a.stride(0)), _c_ll(k), _c_ll(n), _c_ll(0), _c_ll(w.shape[1] * k), _c_ll(0), None, _c_ll(0),
-            _c_int(int(glu is not None)), _c_float(limit), _c_float(alpha)))
+            _c_int(int(glu is not None)), _c_float(limit), _c_float(alpha),
+            _c_int(1 if m - w.shape[0] * (tile - 1) <= MFMA_GROUPS_FEW_ROWS else 4)))
         return out
     _check(library().rv_gemm_groups_plain(
         _stream(), _ptr(a), _dt(a), _ptr(w), _dt(w), _ptr(out), _dt(out), _ptr(row_index), _ptr(tile_group), _c_int(0),

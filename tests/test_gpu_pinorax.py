@@ -62,10 +62,10 @@ def test_embedding_adds_the_vector_of_the_position(out_dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("width", [40, 256, 1030])
-def test_residual_mix_keeps_every_layers_result_and_averages_over_depth(dtype, width):
+@pytest.mark.parametrize("width,layers", [(40, 4), (256, 11), (1030, 4), (2048, 19)])
+def test_residual_mix_keeps_every_layers_result_and_averages_over_depth(dtype, width, layers):
     g = torch.Generator().manual_seed(3)
-    rows, layers, mult = 5, 4, 0.6
+    rows, mult = 5, 0.6
     x0 = torch.randn(rows, width, generator=g)
     x = dev(x0.clone())
     history = torch.full((layers + 1, rows, width), float("nan"), device=DEV)
@@ -217,7 +217,7 @@ def test_products_by_head_with_and_without_a_gate(dtype, rows, heads, n, k):
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("tokens,experts,top,width,inner", [(1, 8, 1, 64, 24), (7, 5, 2, 40, 20), (300, 70, 3, 96, 36),
                                                            (65, 3, 3, 100, 50), (130, 2, 1, 72, 8), (33, 4, 2, 256, 200),
-                                                           (16, 1, 1, 32, 72), (17, 9, 4, 128, 64)])
+                                                           (16, 1, 1, 32, 72), (17, 9, 4, 128, 64), (400, 6, 2, 64, 40)])
 def test_experts_chosen_by_the_tokens_id(dtype, tokens, experts, top, width, inner):
     g = torch.Generator().manual_seed(tokens + experts)
     vocab, limit = 53, 0.8
