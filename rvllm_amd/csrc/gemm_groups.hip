@@ -140,26 +140,34 @@ struct GroupsParams {
   int vec_store;
 };
 
-// NT tiles of 16 rows of W a wave: 4 where many tokens share them (a prompt), 1 where the tokens are few and the
-// launch needs every wave it can get to draw the memory's rate (decoding).  The loop over k is written out UNROLL
-// steps at a time with every read of the steps asked for before the first product, so that a wave has a dozen
-// 16-byte reads in flight.
-template <int NT, bool GLU>
+// A wave takes MT tiles of 16 tokens against NT tiles of 16 rows of W: every value it reads feeds MT or NT
+// products.  Where the tokens are few (decoding) MT = NT = 1, so that a launch has every wave it can get to draw
+// the memory's rate; where they are many (a prompt) MT = 4 and NT = 4 (2 gate and 2 up tiles with GLU), 16
+// products for 8 reads, and the block's four waves share their tokens' values through the CU's cache.  A tile of
+// rows (an entry of tile_group) is 16 MT rows.  The loop over k is written out UNROLL steps at a time with every
+// read of the steps asked for before the first product, so that a wave has a dozen 16-byte reads in flight.
+template <int MT, int NT, bool GLU>
 __global__ void __launch_bounds__(256) gemm_groups_mfma_kernel(const GroupsParams P) {
-  constexpr int UNROLL = NT * (GLU ? 2 : 1) >= 4 ? 2 : 4;
+  constexpr int UNROLL = (MT + NT * (GLU ? 2 : 1)) >= 5 ? 2 : 4;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r16 = lane & 15, kb = lane >> 4;
   const int group = P.tile_group ? P.tile_group[blockIdx.y] : (int)blockIdx.z;
   if (group < 0) return;  // the whole block alike
-  const int m0 = blockIdx.y * 16;
+  const int m0 = blockIdx.y * 16 * MT;
   const int n0 = (blockIdx.x * 4 + wave) * 16 * NT;
   if (n0 >= P.N) return;  // the whole wave
   const uint16_t* a = P.a + (size_t)group * P.a_group_stride;
   const uint16_t* w = P.w + (size_t)group * P.w_group_stride;
-  const int am = m0 + r16;
-  long long a_row = -1;
-  if (am < P.M) a_row = P.row_index ? P.row_index[am] : am;
-  const uint16_t* xr = a + (size_t)(a_row >= 0 ? a_row : 0) * P.lda;
+  const uint16_t* xr[MT];
+  bool x_there[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    const int am = m0 + mt * 16 + r16;
+    long long a_row = -1;
+    if (am < P.M) a_row = P.row_index ? P.row_index[am] : am;
+    x_there[mt] = a_row >= 0;
+    xr[mt] = a + (size_t)(a_row >= 0 ? a_row : 0) * P.lda;
+  }
   const uint16_t* wr[NT];
 #pragma unroll
   for (int t = 0; t < NT; ++t) {
@@ -168,19 +176,22 @@ __global__ void __launch_bounds__(256) gemm_groups_mfma_kernel(const GroupsParam
     wr[t] = w + (size_t)n * P.ldw;
   }
   const size_t up_rows = (size_t)P.N * P.ldw;  // GLU: the up rows follow the N gate rows
-  gg_f32x4 acc[NT], acc_up[NT];
+  gg_f32x4 acc[MT][NT], acc_up[MT][NT];
 #pragma unroll
-  for (int t = 0; t < NT; ++t) {
-    acc[t] = (gg_f32x4){0.f, 0.f, 0.f, 0.f};
-    acc_up[t] = (gg_f32x4){0.f, 0.f, 0.f, 0.f};
-  }
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+      acc[mt][t] = (gg_f32x4){0.f, 0.f, 0.f, 0.f};
+      acc_up[mt][t] = (gg_f32x4){0.f, 0.f, 0.f, 0.f};
+    }
   for (int k0 = 0; k0 < P.K; k0 += 32 * UNROLL) {
-    GgFrag8 xf[UNROLL], wf[UNROLL][NT], uf[UNROLL][NT];
+    GgFrag8 xf[UNROLL][MT], wf[UNROLL][NT], uf[UNROLL][NT];
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
       const int k = k0 + u * 32 + kb * 8;
       const int kk = k < P.K ? k : 0;  // reads are unconditional, from an address that exists; what lies past K is zeroed
-      xf[u].u4 = *(const uint4*)(xr + kk);
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) xf[u][mt].u4 = *(const uint4*)(xr[mt] + kk);
 #pragma unroll
       for (int t = 0; t < NT; ++t) {
         wf[u][t].u4 = *(const uint4*)(wr[t] + kk);
@@ -189,55 +200,64 @@ __global__ void __launch_bounds__(256) gemm_groups_mfma_kernel(const GroupsParam
     }
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
-      if (k0 + u * 32 + kb * 8 >= P.K || a_row < 0) xf[u].u4 = make_uint4(0, 0, 0, 0);
+      const bool past = k0 + u * 32 + kb * 8 >= P.K;
 #pragma unroll
-      for (int t = 0; t < NT; ++t) {
-        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[u][t].v, xf[u].v, acc[t], 0, 0, 0);
-        if constexpr (GLU) acc_up[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(uf[u][t].v, xf[u].v, acc_up[t], 0, 0, 0);
+      for (int mt = 0; mt < MT; ++mt) {
+        if (past || !x_there[mt]) xf[u][mt].u4 = make_uint4(0, 0, 0, 0);
+#pragma unroll
+        for (int t = 0; t < NT; ++t) {
+          acc[mt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[u][t].v, xf[u][mt].v, acc[mt][t], 0, 0, 0);
+          if constexpr (GLU)
+            acc_up[mt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(uf[u][t].v, xf[u][mt].v, acc_up[mt][t], 0, 0, 0);
+        }
       }
     }
   }
-  if (am >= P.M) return;
-  uint16_t* cr = P.c + (size_t)group * P.c_group_stride + (size_t)am * P.ldc;
-  const uint16_t* gr = P.gate ? P.gate + (size_t)group * P.c_group_stride + (size_t)am * P.ldg : nullptr;
 #pragma unroll
-  for (int t = 0; t < NT; ++t) {
-    const int n = n0 + t * 16 + kb * 4;
-    float v[4];
+  for (int mt = 0; mt < MT; ++mt) {
+    const int am = m0 + mt * 16 + r16;
+    if (am >= P.M) continue;
+    uint16_t* cr = P.c + (size_t)group * P.c_group_stride + (size_t)am * P.ldc;
+    const uint16_t* gr = P.gate ? P.gate + (size_t)group * P.c_group_stride + (size_t)am * P.ldg : nullptr;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      v[i] = acc[t][i];
-      if constexpr (GLU) {
-        const float g = fminf(v[i], P.limit);
-        const float u = fminf(fmaxf(acc_up[t][i], -P.limit), P.limit);
-        v[i] = g * (u + 1.0f) * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * P.alpha * g));
+    for (int t = 0; t < NT; ++t) {
+      const int n = n0 + t * 16 + kb * 4;
+      float v[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        v[i] = acc[mt][t][i];
+        if constexpr (GLU) {
+          const float g = fminf(v[i], P.limit);
+          const float u = fminf(fmaxf(acc_up[mt][t][i], -P.limit), P.limit);
+          v[i] = g * (u + 1.0f) * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * P.alpha * g));
+        }
+        if (gr != nullptr && n + i < P.N) {
+          const float z = __uint_as_float(((uint32_t)gr[n + i]) << 16);
+          v[i] *= __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * z));
+        }
       }
-      if (gr != nullptr && n + i < P.N) {
-        const float z = __uint_as_float(((uint32_t)gr[n + i]) << 16);
-        v[i] *= __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * z));
-      }
-    }
-    if (P.vec_store && n + 3 < P.N) {
-      uint2 packed;
-      packed.x = rv_pack_bf16x2(v[0], v[1]);
-      packed.y = rv_pack_bf16x2(v[2], v[3]);
-      *(uint2*)(cr + n) = packed;
-    } else {
+      if (P.vec_store && n + 3 < P.N) {
+        uint2 packed;
+        packed.x = rv_pack_bf16x2(v[0], v[1]);
+        packed.y = rv_pack_bf16x2(v[2], v[3]);
+        *(uint2*)(cr + n) = packed;
+      } else {
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
-        if (n + i < P.N) cr[n + i] = rv_f32_to_bf16_bits(v[i]);
+        for (int i = 0; i < 4; ++i)
+          if (n + i < P.N) cr[n + i] = rv_f32_to_bf16_bits(v[i]);
+      }
     }
   }
 }
 
 // bf16 everywhere.  N: columns of C; with `glu` w holds 2 N rows a group.  groups > 0: the heads' form; 0: the
-// experts' form with tiles of 16 rows.  K, the leading dimensions of a and w and the group strides of a and w must
+// experts' form with tiles of 16 * token_tiles rows.  token_tiles: 1 (few rows) or 4 (many).  K, the leading dimensions of a and w and the group strides of a and w must
 // be multiples of 8 and a, w lie on 16-byte boundaries (a lane reads 16 bytes at a time).
 extern "C" int rv_gemm_groups_mfma(hipStream_t stream, const void* a, const void* w, void* c, const int* row_index,
                                    const int* tile_group, int groups, int M, int N, int K, long long lda,
                                    long long ldw, long long ldc, long long a_group_stride, long long w_group_stride,
                                    long long c_group_stride, const void* gate, long long ldg, int glu, float limit,
-                                   float alpha, int tiles_a_wave) {
+                                   float alpha, int token_tiles) {
   RV_CHECK(M >= 0 && N > 0 && K > 0 && groups >= 0, "gemm_groups_mfma: bad sizes M=%d N=%d K=%d groups=%d", M, N, K, groups);
   RV_CHECK((groups > 0) == (tile_group == nullptr), "gemm_groups_mfma: either a number of groups or the groups of the row tiles");
   RV_CHECK(K % 8 == 0 && lda % 8 == 0 && ldw % 8 == 0 && a_group_stride % 8 == 0 && w_group_stride % 8 == 0 &&
@@ -246,7 +266,7 @@ extern "C" int rv_gemm_groups_mfma(hipStream_t stream, const void* a, const void
            "16-byte aligned");
   RV_CHECK(lda >= K && ldw >= K && ldc >= N && (gate == nullptr || ldg >= N), "gemm_groups_mfma: rows too short");
   RV_CHECK(!glu || (gate == nullptr && limit > 0.f), "gemm_groups_mfma: the gated activation takes a limit and no gate");
-  RV_CHECK(tiles_a_wave == 1 || tiles_a_wave == 4, "gemm_groups_mfma: 1 or 4 tiles of rows a wave, not %d", tiles_a_wave);
+  RV_CHECK(token_tiles == 1 || token_tiles == 4, "gemm_groups_mfma: 1 or 4 tiles of 16 tokens a wave, not %d", token_tiles);
   if (M == 0) return 0;
   GroupsParams P;
   P.a = (const uint16_t*)a;
@@ -260,12 +280,13 @@ extern "C" int rv_gemm_groups_mfma(hipStream_t stream, const void* a, const void
   P.a_group_stride = a_group_stride, P.w_group_stride = w_group_stride, P.c_group_stride = c_group_stride;
   P.limit = limit, P.alpha = alpha;
   P.vec_store = (ldc % 4 == 0 && c_group_stride % 4 == 0 && ((uintptr_t)c & 7) == 0) ? 1 : 0;
-  dim3 grid(rv_div_up(N, 16 * tiles_a_wave * 4), rv_div_up(M, 16), groups > 0 ? groups : 1), block(256);
+  const int rows_of_w = token_tiles == 1 ? 16 : (glu ? 32 : 64);  // of a wave
+  dim3 grid(rv_div_up(N, rows_of_w * 4), rv_div_up(M, 16 * token_tiles), groups > 0 ? groups : 1), block(256);
   RV_CHECK(grid.y < 65536 && grid.z < 65536, "gemm_groups_mfma: too many row tiles or groups for one launch");
-  if (glu && tiles_a_wave == 1) gemm_groups_mfma_kernel<1, true><<<grid, block, 0, stream>>>(P);
-  else if (glu) gemm_groups_mfma_kernel<4, true><<<grid, block, 0, stream>>>(P);
-  else if (tiles_a_wave == 1) gemm_groups_mfma_kernel<1, false><<<grid, block, 0, stream>>>(P);
-  else gemm_groups_mfma_kernel<4, false><<<grid, block, 0, stream>>>(P);
+  if (glu && token_tiles == 1) gemm_groups_mfma_kernel<1, 1, true><<<grid, block, 0, stream>>>(P);
+  else if (glu) gemm_groups_mfma_kernel<4, 2, true><<<grid, block, 0, stream>>>(P);
+  else if (token_tiles == 1) gemm_groups_mfma_kernel<1, 1, false><<<grid, block, 0, stream>>>(P);
+  else gemm_groups_mfma_kernel<4, 4, false><<<grid, block, 0, stream>>>(P);
   RV_LAUNCH_CHECK("gemm_groups_mfma");
   return 0;
 }

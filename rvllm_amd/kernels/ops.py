@@ -336,8 +336,9 @@ def gemm_heads(a: torch.Tensor, a_col0: int, w: torch.Tensor, out: Optional[torc
     return out
 
 
-# Up to this many rows a wave of the matrix-core kernel for products by group takes one tile of 16 rows of the
-# matrix, so that a launch has waves enough to draw the memory's rate; beyond, four, which share the rows' values.
+# Up to this many rows a wave of the matrix-core kernel for products by group takes one tile of 16 rows against
+# one tile of 16 rows of the matrix, so that a launch has waves enough to draw the memory's rate; beyond, four tiles
+# of rows against four of the matrix, so that every value read feeds four products.
 MFMA_GROUPS_FEW_ROWS = 256
 
 
@@ -346,16 +347,17 @@ def _mfma_groups_take(aptr: int, lda: int, w: torch.Tensor, k: int) -> bool:
     return k % 8 == 0 and lda % 8 == 0 and aptr % 16 == 0 and w.data_ptr() % 16 == 0
 
 
-MOE_TILE_ROWS = 64  # rows of one expert that a block of the 32-bit grouped product takes
-MOE_TILE_ROWS_MFMA = 16  # and a wave of the matrix-core one
+MOE_TILE_ROWS = 64  # rows of one expert that a block of the grouped products takes
+MOE_TILE_ROWS_FEW = 16  # the matrix-core kernel's tiles while a step's rows are few
 
 
-def moe_tile_rows(dtype: torch.dtype, *inner_sizes: int) -> int:
-    """The rows a tile of the sorted order holds for products of this type whose summed sizes are
-    ``inner_sizes``: 16 where the matrix-core kernel takes them (bf16, sizes that are multiples of 8), else 64."""
-    if dtype == torch.bfloat16 and all(k % 8 == 0 for k in inner_sizes):
-        return MOE_TILE_ROWS_MFMA
-    return MOE_TILE_ROWS
+def moe_plan(dtype: torch.dtype, rows: int, *inner_sizes: int) -> tuple[int, bool]:
+    """(rows a tile of the sorted order holds, whether the matrix-core kernel multiplies) for a step of ``rows``
+    (token, choice) pairs and products whose summed sizes are ``inner_sizes``: bf16 with sizes that are multiples
+    of 8 runs on the matrix cores, in tiles of 16 rows while the rows are few and of 64 beyond; everything else in
+    tiles of 64 rows on the 32-bit kernel."""
+    mfma = dtype == torch.bfloat16 and all(k % 8 == 0 for k in inner_sizes)
+    return (MOE_TILE_ROWS_FEW if mfma and rows <= MFMA_GROUPS_FEW_ROWS else MOE_TILE_ROWS), mfma
 
 
 def moe_capacity(num_tokens: int, top: int, experts: int, tile: int = MOE_TILE_ROWS) -> int:
@@ -383,18 +385,18 @@ def moe_route(token_ids: torch.Tensor, num_tokens: int, table: torch.Tensor, exp
 
 
 def gemm_experts(a: torch.Tensor, w: torch.Tensor, tile_group: torch.Tensor, row_index: Optional[torch.Tensor] = None,
-                 out: Optional[torch.Tensor] = None, tile: int = MOE_TILE_ROWS,
+                 out: Optional[torch.Tensor] = None, tile: int = MOE_TILE_ROWS, mfma: bool = False,
                  glu: Optional[tuple[float, float]] = None) -> torch.Tensor:
     """``out[r] = a[row_index[r]] @ w[tile_group[r // tile]]^T`` for the sorted rows of ``moe_route``; ``w`` is
     ``[experts, N, K]``.  Without ``row_index`` the rows of ``a`` are the sorted rows themselves.  Rows of tiles
-    without an expert are left as they are.  ``tile`` is the route's (``moe_tile_rows``): 16 runs the matrix-core
-    kernel, 64 the 32-bit one.  ``glu`` = (limit, alpha), with tiles of 16 only: ``w`` holds each expert's gate rows
-    and then its up rows, and the result is the clamped gated activation of the two products, ``[rows, N / 2]``."""
+    without an expert are left as they are.  ``tile`` and ``mfma`` are the step's plan (``moe_plan``).  ``glu`` =
+    (limit, alpha), on the matrix cores only: ``w`` holds each expert's gate rows and then its up rows, and the
+    result is the clamped gated activation of the two products, ``[rows, N / 2]``."""
     _gpu(a, w, tile_group, row_index, out)
     _i32(tile_group)
     _need(a.dim() == 2 and w.dim() == 3 and a.dtype == w.dtype and a.dtype in _DT and a.shape[1] == w.shape[2],
           "gemm_experts: rows [*, K] against matrices [experts, N, K] of one type expected")
-    _need(tile in (MOE_TILE_ROWS, MOE_TILE_ROWS_MFMA), f"gemm_experts: tiles of {tile} rows")
+    _need(tile == MOE_TILE_ROWS or (mfma and tile == MOE_TILE_ROWS_FEW), f"gemm_experts: tiles of {tile} rows")
     m = tile_group.numel() * tile
     if row_index is not None:
         _i32(row_index)
@@ -403,20 +405,19 @@ def gemm_experts(a: torch.Tensor, w: torch.Tensor, tile_group: torch.Tensor, row
         _need(a.shape[0] == m, "gemm_experts: the rows must be the sorted rows")
     _, n, k = w.shape
     if glu is not None:
-        _need(n % 2 == 0 and tile == MOE_TILE_ROWS_MFMA, "gemm_experts: the activation is applied by the matrix-core kernel")
+        _need(n % 2 == 0 and mfma, "gemm_experts: the activation is applied by the matrix-core kernel")
         n //= 2
     if out is None:
         out = torch.empty((m, n), dtype=a.dtype, device=a.device)
     _need(out.shape == (m, n) and out.dtype == a.dtype, "gemm_experts: bad out")
-    if tile == MOE_TILE_ROWS_MFMA:
+    if mfma:
         _need(a.dtype == torch.bfloat16 and _mfma_groups_take(a.data_ptr(), a.stride(0), w, k),
-              "gemm_experts: tiles of 16 rows are the matrix-core kernel's: bf16, sizes that are multiples of 8")
+              "gemm_experts: the matrix-core kernel takes bf16 and sizes that are multiples of 8")
         limit, alpha = glu if glu is not None else (0.0, 0.0)
         _check(library().rv_gemm_groups_mfma(
             _stream(), _ptr(a), _ptr(w), _ptr(out), _ptr(row_index), _ptr(tile_group), _c_int(0), _c_int(m), _c_int(n),
             _c_int(k), _c_ll(a.stride(0)), _c_ll(k), _c_ll(n), _c_ll(0), _c_ll(w.shape[1] * k), _c_ll(0), None, _c_ll(0),
-            _c_int(int(glu is not None)), _c_float(limit), _c_float(alpha),
-            _c_int(1 if m - w.shape[0] * (tile - 1) <= MFMA_GROUPS_FEW_ROWS else 4)))
+            _c_int(int(glu is not None)), _c_float(limit), _c_float(alpha), _c_int(tile // 16)))
         return out
     _check(library().rv_gemm_groups_plain(
         _stream(), _ptr(a), _dt(a), _ptr(w), _dt(w), _ptr(out), _dt(out), _ptr(row_index), _ptr(tile_group), _c_int(0),

@@ -102,15 +102,15 @@ class RoutedExperts(FeedForward):
         if self.shared is not None:
             act = ops.clamped_glu(linear(x, self.shared_gate_up), self.shared["limit"], self.shared["alpha"])
             shared = linear(act, self.shared_down)
-        tile = ops.moe_tile_rows(x.dtype, self.hidden_size, self.intermediate_size)
+        tile, mfma = ops.moe_plan(x.dtype, n * self.top, self.hidden_size, self.intermediate_size)
         slot_of, row_token, tile_group = ops.moe_route(step.token_ids, n, self.table, self.num_experts, tile)
-        if tile == ops.MOE_TILE_ROWS_MFMA:  # bf16: the product of gates and ups applies the activation itself
-            act = ops.gemm_experts(x, self.w_gate_up, tile_group, row_index=row_token, tile=tile,
+        if mfma:  # bf16: the product of gates and ups applies the activation itself
+            act = ops.gemm_experts(x, self.w_gate_up, tile_group, row_index=row_token, tile=tile, mfma=True,
                                    glu=(self.limit, self.alpha))
         else:
             gate_up = ops.gemm_experts(x, self.w_gate_up, tile_group, row_index=row_token, tile=tile)
             act = ops.clamped_glu(gate_up, self.limit, self.alpha)
-        y = ops.gemm_experts(act, self.w_down, tile_group, tile=tile)
+        y = ops.gemm_experts(act, self.w_down, tile_group, tile=tile, mfma=mfma)
         return ops.moe_combine(y, slot_of, self.top, 1.0 / self.top, n, shared)
 
 

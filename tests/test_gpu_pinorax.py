@@ -233,8 +233,10 @@ def test_experts_chosen_by_the_tokens_id(dtype, tokens, experts, top, width, inn
     want = PP.routed_ff(h.double(), ids.tolist(), {k: (v.double() if v.is_floating_point() else v) for k, v in w.items()}, "", mlp)
     w_gu = dev(torch.stack([torch.cat([w[f"e{e}.gate"], w[f"e{e}.up"]]) for e in range(experts)]))
     w_down = dev(torch.stack([w[f"e{e}.down"] for e in range(experts)]))
-    tile = ops.moe_tile_rows(dtype, width, inner)  # 16 rows and the matrix cores for bf16 sizes in eights, else 64
-    assert tile == (16 if dtype == torch.bfloat16 and width % 8 == 0 and inner % 8 == 0 else 64)
+    tile, mfma = ops.moe_plan(dtype, tokens * top, width, inner)
+    # bf16 sizes in eights run on the matrix cores, in tiles of 16 rows while the rows are few; all else in 64s
+    assert mfma == (dtype == torch.bfloat16 and width % 8 == 0 and inner % 8 == 0)
+    assert tile == (16 if mfma and tokens * top <= 256 else 64)
     slot_of, row_token, tile_group = ops.moe_route(dev(ids), tokens, dev(table), experts, tile)
     # the sorted order: every choice has a row of its own in a tile of its expert, rows know their tokens
     so, rt, tg = slot_of.cpu().view(tokens, top), row_token.cpu(), tile_group.cpu()
@@ -243,16 +245,16 @@ def test_experts_chosen_by_the_tokens_id(dtype, tokens, experts, top, width, inn
         for c in range(top):
             assert rt[so[t, c]] == t and tg[so[t, c] // tile] == table[ids[t], c]
     assert int((rt >= 0).sum()) == tokens * top
-    if tile == 16:  # the activation inside the product
-        act = ops.gemm_experts(dev(h), w_gu, tile_group, row_index=row_token, tile=tile, glu=(limit, 1.702))
+    if mfma:  # the activation inside the product
+        act = ops.gemm_experts(dev(h), w_gu, tile_group, row_index=row_token, tile=tile, mfma=True, glu=(limit, 1.702))
     else:
         act = ops.clamped_glu(ops.gemm_experts(dev(h), w_gu, tile_group, row_index=row_token, tile=tile), limit, 1.702)
-    got = ops.moe_combine(ops.gemm_experts(act, w_down, tile_group, tile=tile), slot_of, top, 1.0 / top, tokens)
+    got = ops.moe_combine(ops.gemm_experts(act, w_down, tile_group, tile=tile, mfma=mfma), slot_of, top, 1.0 / top, tokens)
     close(got, want, dtype)
-    if tile == 16:  # the same through the kernels that take any size
+    if mfma:  # the same through the kernels that take any size
         s64, r64, t64 = ops.moe_route(dev(ids), tokens, dev(table), experts, 64)
         act = ops.clamped_glu(ops.gemm_experts(dev(h), w_gu, t64, row_index=r64), limit, 1.702)
-        close(ops.moe_combine(ops.gemm_experts(act, w_down, t64), s64, top, 1.0 / top, tokens), want, dtype, "tiles of 64")
+        close(ops.moe_combine(ops.gemm_experts(act, w_down, t64), s64, top, 1.0 / top, tokens), want, dtype, "32-bit kernel")
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
