@@ -547,28 +547,34 @@ extern "C" int rv_gated_act(hipStream_t stream, const void* gu, int slices, long
 // gates and ups lie in halves of a row of gu [rows, 2 * inter] (gate i at i, up i at inter + i).
 // ---------------------------------------------------------------------------
 template <typename T>
-__global__ void clamped_glu_kernel(const T* __restrict__ gu, T* __restrict__ out, int inter, long long total,
-                                   float limit, float alpha) {
+__global__ void clamped_glu_kernel(const void* __restrict__ gu, int slices, long long slice_stride, T* __restrict__ out,
+                                   int inter, long long total, float limit, float alpha) {
   const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
   if (idx >= total) return;
   const long long t = idx / inter;
   const int i = (int)(idx - t * inter);
-  const float gate = fminf(rv_to_float(gu[(size_t)t * 2 * inter + i]), limit);
-  const float up = fminf(fmaxf(rv_to_float(gu[(size_t)t * 2 * inter + inter + i]), -limit), limit);
+  float g[1], u[1];
+  row_load_branch<T, 1>(gu, slices, slice_stride, (size_t)t * 2 * inter + i, g);
+  row_load_branch<T, 1>(gu, slices, slice_stride, (size_t)t * 2 * inter + inter + i, u);
+  const float gate = fminf(g[0], limit);
+  const float up = fminf(fmaxf(u[0], -limit), limit);
   out[idx] = rv_from_float<T>(gate / (1.0f + expf(-alpha * gate)) * (up + 1.0f));
 }
 
-extern "C" int rv_clamped_glu(hipStream_t stream, const void* gu, void* out, int dtype, int rows, int inter,
-                              float limit, float alpha) {
+// `slices` 0: gu holds values of the output's type [rows, 2 * inter]; otherwise 32-bit partial sums
+// [slices][rows][2 * inter], slice_stride elements apart (the K slices of a product), added here in their order.
+extern "C" int rv_clamped_glu(hipStream_t stream, const void* gu, int slices, long long slice_stride, void* out,
+                              int dtype, int rows, int inter, float limit, float alpha) {
   RV_CHECK(rows >= 0 && inter > 0 && limit > 0.f, "clamped_glu: bad arguments rows=%d inter=%d limit=%g", rows, inter,
            (double)limit);
+  RV_CHECK(slices >= 0 && (slices == 0 || slice_stride >= 2ll * rows * inter), "clamped_glu: bad partial sums");
   if (rows == 0) return 0;
   const long long total = (long long)rows * inter;
   dim3 grid(rv_div_up(total, 256)), block(256);
   if (dtype == RV_F32)
-    clamped_glu_kernel<float><<<grid, block, 0, stream>>>((const float*)gu, (float*)out, inter, total, limit, alpha);
+    clamped_glu_kernel<float><<<grid, block, 0, stream>>>(gu, slices, slice_stride, (float*)out, inter, total, limit, alpha);
   else if (dtype == RV_BF16)
-    clamped_glu_kernel<bf16_t><<<grid, block, 0, stream>>>((const bf16_t*)gu, (bf16_t*)out, inter, total, limit, alpha);
+    clamped_glu_kernel<bf16_t><<<grid, block, 0, stream>>>(gu, slices, slice_stride, (bf16_t*)out, inter, total, limit, alpha);
   else
     return rv_fail("clamped_glu: unsupported dtype %d", dtype);
   RV_LAUNCH_CHECK("clamped_glu");

@@ -76,31 +76,46 @@ extern "C" int rv_moe_route(hipStream_t stream, const int* token_ids, int num_to
 
 template <typename T>
 __global__ void moe_combine_kernel(const T* __restrict__ y, const int* __restrict__ slot_of, int top, float weight,
-                                   const T* __restrict__ shared, T* __restrict__ out, int width) {
+                                   const void* __restrict__ shared, int shared_slices, long long shared_stride,
+                                   T* __restrict__ out, int width) {
   const int t = blockIdx.x;
   for (int i = threadIdx.x; i < width; i += blockDim.x) {
+    const size_t at = (size_t)t * width + i;
     float acc = 0.f;
     for (int k = 0; k < top; ++k) {
       const int row = slot_of[(size_t)t * top + k];
       if (row >= 0) acc += rv_to_float(y[(size_t)row * width + i]);
     }
     acc *= weight;
-    if (shared != nullptr) acc += rv_to_float(shared[(size_t)t * width + i]);
-    out[(size_t)t * width + i] = rv_from_float<T>(acc);
+    if (shared != nullptr) {
+      if (shared_slices == 0) {
+        acc += rv_to_float(((const T*)shared)[at]);
+      } else {  // the K slices of the shared expert's last product, added in their order, then rounded as stored
+        float sum = 0.f;
+        for (int s = 0; s < shared_slices; ++s) sum += ((const float*)shared)[(size_t)s * shared_stride + at];
+        acc += rv_round_to<T>(sum);
+      }
+    }
+    out[at] = rv_from_float<T>(acc);
   }
 }
 
+// shared: null, values of type `dtype` [tokens, width] (shared_slices 0), or 32-bit partial sums
+// [shared_slices][tokens][width], shared_stride elements apart.
 extern "C" int rv_moe_combine(hipStream_t stream, const void* y, const int* slot_of, int top, float weight,
-                              const void* shared, void* out, int dtype, int num_tokens, int width) {
+                              const void* shared, int shared_slices, long long shared_stride, void* out, int dtype,
+                              int num_tokens, int width) {
   RV_CHECK(num_tokens >= 0 && width > 0 && top > 0, "moe_combine: bad sizes tokens=%d width=%d top=%d", num_tokens, width, top);
+  RV_CHECK(shared_slices >= 0 && (shared_slices == 0 || shared_stride >= (long long)num_tokens * width),
+           "moe_combine: bad partial sums");
   if (num_tokens == 0) return 0;
   dim3 grid(num_tokens), block(256);
   if (dtype == RV_F32)
-    moe_combine_kernel<float><<<grid, block, 0, stream>>>((const float*)y, slot_of, top, weight, (const float*)shared,
-                                                          (float*)out, width);
+    moe_combine_kernel<float><<<grid, block, 0, stream>>>((const float*)y, slot_of, top, weight, shared, shared_slices,
+                                                          shared_stride, (float*)out, width);
   else if (dtype == RV_BF16)
-    moe_combine_kernel<bf16_t><<<grid, block, 0, stream>>>((const bf16_t*)y, slot_of, top, weight,
-                                                           (const bf16_t*)shared, (bf16_t*)out, width);
+    moe_combine_kernel<bf16_t><<<grid, block, 0, stream>>>((const bf16_t*)y, slot_of, top, weight, shared,
+                                                           shared_slices, shared_stride, (bf16_t*)out, width);
   else
     return rv_fail("moe_combine: unsupported dtype %d", dtype);
   RV_LAUNCH_CHECK("moe_combine");

@@ -426,30 +426,34 @@ def gemm_experts(a: torch.Tensor, w: torch.Tensor, tile_group: torch.Tensor, row
     return out
 
 
-def moe_combine(y: torch.Tensor, slot_of: torch.Tensor, top: int, weight: float, num_tokens: int,
-                shared: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """out[t] = weight * sum_k y[slot_of[t * top + k]] (+ shared[t])."""
-    _gpu(y, slot_of, shared)
+def moe_combine(y: torch.Tensor, slot_of: torch.Tensor, top: int, weight: float, num_tokens: int, shared=None) -> torch.Tensor:
+    """out[t] = weight * sum_k y[slot_of[t * top + k]] (+ shared[t]); ``shared`` is a tensor or unreduced
+    ``SlicedSums``."""
+    _gpu(y, slot_of)
     _i32(slot_of)
     width = y.shape[1]
     _need(slot_of.numel() == num_tokens * top, "moe_combine: one sorted row for every choice")
-    _need(shared is None or (shared.shape == (num_tokens, width) and shared.dtype == y.dtype),
-          "moe_combine: the shared expert's output must match")
+    sptr, s_slices, s_stride = None, 0, 0
+    if shared is not None:
+        sptr, s_slices, s_stride, s_rows, s_width, s_dtype = _branch_args(shared, "moe_combine")
+        _need((s_rows, s_width) == (num_tokens, width) and s_dtype == y.dtype,
+              "moe_combine: the shared expert's output must match")
     out = torch.empty((num_tokens, width), dtype=y.dtype, device=y.device)
-    _check(library().rv_moe_combine(_stream(), _ptr(y), _ptr(slot_of), _c_int(top), _c_float(weight), _ptr(shared),
-                                    _ptr(out), _dt(out), _c_int(num_tokens), _c_int(width)))
+    _check(library().rv_moe_combine(_stream(), _ptr(y), _ptr(slot_of), _c_int(top), _c_float(weight), sptr,
+                                    _c_int(s_slices), _c_ll(s_stride), _ptr(out), _dt(out), _c_int(num_tokens),
+                                    _c_int(width)))
     return out
 
 
-def clamped_glu(gate_up: torch.Tensor, limit: float, alpha: float) -> torch.Tensor:
+def clamped_glu(gate_up, limit: float, alpha: float) -> torch.Tensor:
     """g = min(gate, limit), u = clamp(up, -limit, limit): out = g * sigmoid(alpha g) * (u + 1); gates and ups lie in
-    the halves of a row of ``gate_up [rows, 2 I]``."""
-    _gpu(gate_up)
-    _need(gate_up.dim() == 2 and gate_up.shape[1] % 2 == 0, "clamped_glu: rows of gates and ups expected")
-    rows, inter = gate_up.shape[0], gate_up.shape[1] // 2
-    out = torch.empty((rows, inter), dtype=gate_up.dtype, device=gate_up.device)
-    _check(library().rv_clamped_glu(_stream(), _ptr(gate_up), _ptr(out), _dt(out), _c_int(rows), _c_int(inter),
-                                    _c_float(limit), _c_float(alpha)))
+    the halves of a row of ``gate_up [rows, 2 I]``, a tensor or unreduced ``SlicedSums``."""
+    gptr, slices, stride, rows, two_i, dtype = _branch_args(gate_up, "clamped_glu")
+    _need(two_i % 2 == 0, "clamped_glu: rows of gates and ups expected")
+    inter = two_i // 2
+    out = torch.empty((rows, inter), dtype=dtype, device=gate_up.device)
+    _check(library().rv_clamped_glu(_stream(), gptr, _c_int(slices), _c_ll(stride), _ptr(out), _dt(out), _c_int(rows),
+                                    _c_int(inter), _c_float(limit), _c_float(alpha)))
     return out
 
 

@@ -100,8 +100,10 @@ class RoutedExperts(FeedForward):
         n = x.shape[0]
         shared = None
         if self.shared is not None:
-            act = ops.clamped_glu(linear(x, self.shared_gate_up), self.shared["limit"], self.shared["alpha"])
-            shared = linear(act, self.shared_down)
+            # products of few rows stay unreduced K slices; the kernels that take them add them up
+            act = ops.clamped_glu(linear(x, self.shared_gate_up, sliced_ok=True), self.shared["limit"],
+                                  self.shared["alpha"])
+            shared = linear(act, self.shared_down, sliced_ok=True)
         tile, mfma = ops.moe_plan(x.dtype, n * self.top, self.hidden_size, self.intermediate_size)
         slot_of, row_token, tile_group = ops.moe_route(step.token_ids, n, self.table, self.num_experts, tile)
         if mfma:  # bf16: the product of gates and ups applies the activation itself
