@@ -719,10 +719,22 @@ def attention_wave_slots(head_dim: int) -> int:
     return slots if slots > 0 else _ATTN_WAVE_SLOTS_FALLBACK
 
 
+def shared_head_groups(num_q_heads: int, cache_kv_heads: int) -> int:
+    """How many groups the query heads form for the matrix-core attention kernels.  Usually one group a key/value
+    head.  Where the cache holds a single head that more than 16 query heads share (latent attention), the heads are
+    cut into equal groups of at most 16, each of which reads that one head: the largest divisor of the head count
+    that a tile holds."""
+    if cache_kv_heads != 1 or num_q_heads <= MFMA_ATTENTION_MAX_GROUP:
+        return cache_kv_heads
+    group = max(g for g in range(1, MFMA_ATTENTION_MAX_GROUP + 1) if num_q_heads % g == 0)
+    return num_q_heads // group
+
+
 def mfma_attention_covers(k_pages: torch.Tensor, v_pages: torch.Tensor, num_q_heads: int) -> bool:
     _, nkv, page_size, hd = k_pages.shape
-    return (hd % 16 == 0 and hd <= MFMA_ATTENTION_MAX_HEAD_DIM and page_size % 16 == 0
-            and num_q_heads % nkv == 0 and num_q_heads // nkv <= MFMA_ATTENTION_MAX_GROUP)
+    if not (hd % 16 == 0 and hd <= MFMA_ATTENTION_MAX_HEAD_DIM and page_size % 16 == 0 and num_q_heads % nkv == 0):
+        return False
+    return num_q_heads // shared_head_groups(num_q_heads, nkv) <= MFMA_ATTENTION_MAX_GROUP
 
 
 @functools.lru_cache(maxsize=4096)
@@ -948,6 +960,7 @@ def paged_attention_mfma(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.
     _need(q.shape == (n, num_q_heads * hd) and out.shape == q.shape and out.dtype == q.dtype,
           "attention (matrix cores): bad q or out shape")
     _need(n == step.num_tokens, "attention (matrix cores): q must hold the step's tokens")
+    cache_nkv, nkv = nkv, shared_head_groups(num_q_heads, nkv)  # groups of query heads; they may share the cache's head
     group = num_q_heads // nkv
     group_pad = 1
     while group_pad < group:
@@ -982,7 +995,7 @@ def paged_attention_mfma(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.
                      _c_int(block_table.shape[1]), _ptr(step.q_start), _ptr(step.chunk_start), _ptr(out), _c_int(n),
                      _c_int(step.num_requests), _c_int(tiles), _c_int(num_q_heads), _c_int(nkv), _c_int(hd),
                      _c_int(page_size), _c_int(num_pages), _c_int(window or 0), _c_int(portion_min), _c_float(scale),
-                     _c_int(piece_max), _c_int(pieces_max), _ptr(part), _ptr(sinks)))
+                     _c_int(piece_max), _c_int(pieces_max), _ptr(part), _ptr(sinks), _c_int(cache_nkv)))
     if shortest_rest > 0:
         tiles, num_splits, split_len = plan_attention_splits(step.num_requests, shortest_rest, step.max_context, nkv,
                                                              group, window, hd, attention_wave_slots(hd))
@@ -1011,7 +1024,8 @@ def paged_attention_mfma(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.
                      _ptr(out), _ptr(part_o), _ptr(part_ml), _c_int(n), _c_int(step.num_requests), _c_int(tiles),
                      _c_int(num_q_heads), _c_int(nkv), _c_int(hd), _c_int(page_size), _c_int(num_pages),
                      _c_int(window or 0), _c_int(num_splits), _c_int(split_len),
-                     _c_int(portion_min - 1 if use_prefill else 0), _c_int(block_cols), _c_float(scale), _ptr(sinks)))
+                     _c_int(portion_min - 1 if use_prefill else 0), _c_int(block_cols), _c_float(scale), _ptr(sinks),
+                     _c_int(cache_nkv)))
     return out
 
 

@@ -5,7 +5,7 @@ dim^-1/2, a multiplier of 1, layers without a feed-forward or without a shared e
 P  four layers, every layer its own head sizes: experts (2 of 5, shared), dense, none, experts (3 of 3, no shared);
    ranks that are multiples of 16, so bf16 attention runs on the matrix cores
 Q  widths that are no multiple of 8, a rank of 40 and 17 heads: bf16 takes the kernels for any size
-R  layers wide enough for long sequences: far keys, page borders
+R  layers wide enough for long sequences: far keys, page borders; 20 heads in a layer (two groups over one cached head)
 """
 
 from __future__ import annotations
@@ -55,7 +55,7 @@ CONFIG_R = {
     "residual_mult": 0.4, "logit_softcap": 20.0,
     "layers": [
         _layer(_mixer(8, 32, 32, 128, 0.2), _moe(16, 2, 64, 1.5, {"ff": 64, "limit": 1.0})),
-        _layer(_mixer(4, 64, 48, 64, 0.15), {"kind": "dense", "ff": 320}),
+        _layer(_mixer(20, 16, 24, 64, 0.15), {"kind": "dense", "ff": 320}),
     ],
 }
 
