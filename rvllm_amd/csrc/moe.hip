@@ -92,7 +92,14 @@ __global__ void moe_combine_kernel(const T* __restrict__ y, const int* __restric
         acc += rv_to_float(((const T*)shared)[at]);
       } else {  // the K slices of the shared expert's last product, added in their order, then rounded as stored
         float sum = 0.f;
-        for (int s = 0; s < shared_slices; ++s) sum += ((const float*)shared)[(size_t)s * shared_stride + at];
+        const float* p = (const float*)shared + at;
+        int s = 0;
+        for (; s + 4 <= shared_slices; s += 4) {  // four reads on their way together, added in the slices' order
+          const float q0 = p[(size_t)s * shared_stride], q1 = p[(size_t)(s + 1) * shared_stride];
+          const float q2 = p[(size_t)(s + 2) * shared_stride], q3 = p[(size_t)(s + 3) * shared_stride];
+          sum += q0, sum += q1, sum += q2, sum += q3;
+        }
+        for (; s < shared_slices; ++s) sum += p[(size_t)s * shared_stride];
         acc += rv_round_to<T>(sum);
       }
     }
@@ -109,7 +116,7 @@ extern "C" int rv_moe_combine(hipStream_t stream, const void* y, const int* slot
   RV_CHECK(shared_slices >= 0 && (shared_slices == 0 || shared_stride >= (long long)num_tokens * width),
            "moe_combine: bad partial sums");
   if (num_tokens == 0) return 0;
-  dim3 grid(num_tokens), block(256);
+  dim3 grid(num_tokens), block(width >= 1024 ? 1024 : (width > 256 ? 512 : 256));  // few rows: a row's reads side by side
   if (dtype == RV_F32)
     moe_combine_kernel<float><<<grid, block, 0, stream>>>((const float*)y, slot_of, top, weight, shared, shared_slices,
                                                           shared_stride, (float*)out, width);
