@@ -134,3 +134,15 @@ def test_plain_depth_average_and_layers_without_a_feed_forward(tmp_path):
     assert torch.allclose(PP.depth_average([torch.ones(2), 3 * torch.ones(2)], torch.tensor([0.5, 0.25])), torch.full((2,), 1.25))
     # prefixes give the same logits: the model is causal
     assert torch.allclose(PP.forward(weights, cfg, [5, 6, 7]), logits[:3])
+
+
+def test_the_command_line_takes_the_design_from_a_folder_or_a_configuration(tmp_path, capsys):
+    from rvllm_amd import cli
+
+    (tmp_path / "config.json").write_text(json.dumps(tiny_pinorax.CONFIG_Q))
+    assert cli.main(["--model", str(tmp_path), "--dry-run", "--prompt-ids", "1 2 96"], {}) == 0
+    assert json.loads(capsys.readouterr().out)["architecture"] == "Pinorax"
+    assert cli.main(["--model", str(tmp_path), "--dry-run", "--prompt-ids", "1 97"], {}) == 2  # outside the vocabulary
+    capsys.readouterr()
+    assert cli.main(["--random-weights", str(tmp_path / "config.json"), "--dry-run", "--prompt-len", "8"], {}) == 0
+    assert json.loads(capsys.readouterr().out)["architecture"] == "Pinorax"
