@@ -272,6 +272,150 @@ __global__ void __launch_bounds__(256) gemm_groups_mfma_kernel(const GroupsParam
   }
 }
 
+// The experts' products of many rows, tiles staged through LDS.  A block of four waves takes a tile of 64 rows
+// (one entry of tile_group) against 256 rows of its expert's matrix, 64 values of k at a time: the block copies
+// both tiles from memory into LDS once (every row's 128 bytes as one run: eight lanes, 16 bytes each), and every
+// wave multiplies all 64 rows against its 64 rows of the matrix from there, so a value that comes through the
+// memory's caches once feeds four waves' products (read straight into registers, as the kernel above does it, the
+// same product asks the CU's vector cache for 0.5 KB a product tile and keeps the matrix cores busy a tenth of the
+// time).  The next 64 values of k are asked for before this round's products and written to LDS after them.
+// Without GLU a wave's 64 rows of the matrix are 64 columns of C; with GLU they are 32 gate rows and their 32 up
+// rows, and the activation is applied where both sums are held.  Rows of LDS are 16 bytes longer than their data,
+// which spreads a fragment's sixteen rows over the banks.
+#define GL_BM 64
+#define GL_BW 256
+#define GL_BK 64
+#define GL_LD (GL_BK + 8)  // elements a row of LDS
+
+template <bool GLU>
+__global__ void __launch_bounds__(256) gemm_experts_lds_kernel(const GroupsParams P) {
+  __shared__ __attribute__((aligned(16))) uint16_t xs[GL_BM * GL_LD];
+  __shared__ __attribute__((aligned(16))) uint16_t ws[GL_BW * GL_LD];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int r16 = lane & 15, kb = lane >> 4;
+  const int group = P.tile_group[blockIdx.y];
+  if (group < 0) return;  // the whole block alike, before any barrier
+  constexpr int COLS = GLU ? GL_BW / 2 : GL_BW;  // columns of C a block takes
+  const int m0 = blockIdx.y * GL_BM;
+  const int n0 = blockIdx.x * COLS;
+  const uint16_t* w = P.w + (size_t)group * P.w_group_stride;
+
+  // what this thread copies each round: 2 pieces of 16 bytes of the rows' tile, 8 of the matrix's
+  const int piece_k = (tid & 7) * 8;  // its place among a row's 64 values of k
+  const uint16_t* x_src[2];
+  bool x_there[2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int row = (tid >> 3) + i * 32;
+    const int am = m0 + row;
+    long long a_row = -1;
+    if (am < P.M) a_row = P.row_index ? P.row_index[am] : am;
+    x_there[i] = a_row >= 0;
+    x_src[i] = P.a + (size_t)(a_row >= 0 ? a_row : 0) * P.lda + piece_k;
+  }
+  const uint16_t* w_src[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int row = (tid >> 3) + i * 32;  // of the block's 256 rows of the matrix
+    int n;
+    if constexpr (GLU) n = row < COLS ? n0 + row : P.N + n0 + (row - COLS);  // gate rows, then their up rows
+    else n = n0 + row;
+    const int last = GLU ? 2 * P.N - 1 : P.N - 1;
+    n = n < last ? n : last;  // rows past the end repeat the last one; their columns are not stored
+    w_src[i] = w + (size_t)n * P.ldw + piece_k;
+  }
+  uint4 x_reg[2], w_reg[8];
+  auto ask = [&](int k0) {
+    const bool in = k0 + piece_k < P.K;  // K is a multiple of 8: a piece lies inside or outside
+    const int kk = in ? k0 : 0;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      x_reg[i] = *(const uint4*)(x_src[i] + kk);
+      if (!in || !x_there[i]) x_reg[i] = make_uint4(0, 0, 0, 0);
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      w_reg[i] = *(const uint4*)(w_src[i] + kk);
+      if (!in) w_reg[i] = make_uint4(0, 0, 0, 0);
+    }
+  };
+  auto put = [&]() {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) *(uint4*)(xs + ((tid >> 3) + i * 32) * GL_LD + piece_k) = x_reg[i];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) *(uint4*)(ws + ((tid >> 3) + i * 32) * GL_LD + piece_k) = w_reg[i];
+  };
+
+  gg_f32x4 acc[4][4];
+#pragma unroll
+  for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+    for (int t = 0; t < 4; ++t) acc[mt][t] = (gg_f32x4){0.f, 0.f, 0.f, 0.f};
+  // the wave's four tiles of 16 rows of the matrix, as rows of ws
+  int w_row[4];
+#pragma unroll
+  for (int t = 0; t < 4; ++t) {
+    if constexpr (GLU) w_row[t] = (t < 2 ? 0 : COLS) + wave * 32 + (t & 1) * 16;
+    else w_row[t] = wave * 64 + t * 16;
+  }
+
+  ask(0);
+  put();
+  __syncthreads();
+  for (int k0 = 0; k0 < P.K; k0 += GL_BK) {
+    const bool more = k0 + GL_BK < P.K;  // the same for the whole block
+    if (more) ask(k0 + GL_BK);
+#pragma unroll
+    for (int ks = 0; ks < GL_BK / 32; ++ks) {
+      GgFrag8 xf[4], wf[4];
+#pragma unroll
+      for (int mt = 0; mt < 4; ++mt) xf[mt].u4 = *(const uint4*)(xs + (mt * 16 + r16) * GL_LD + ks * 32 + kb * 8);
+#pragma unroll
+      for (int t = 0; t < 4; ++t) wf[t].u4 = *(const uint4*)(ws + (w_row[t] + r16) * GL_LD + ks * 32 + kb * 8);
+#pragma unroll
+      for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+          acc[mt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[t].v, xf[mt].v, acc[mt][t], 0, 0, 0);
+    }
+    __syncthreads();  // every wave has read this round's tiles
+    if (more) put();
+    __syncthreads();
+  }
+
+  constexpr int OUT_TILES = GLU ? 2 : 4;
+#pragma unroll
+  for (int mt = 0; mt < 4; ++mt) {
+    const int am = m0 + mt * 16 + r16;
+    if (am >= P.M) continue;
+    uint16_t* cr = P.c + (size_t)am * P.ldc;
+#pragma unroll
+    for (int t = 0; t < OUT_TILES; ++t) {
+      const int n = n0 + (GLU ? wave * 32 : wave * 64) + t * 16 + kb * 4;
+      float v[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        v[i] = acc[mt][t][i];
+        if constexpr (GLU) {
+          const float g = fminf(v[i], P.limit);
+          const float u = fminf(fmaxf(acc[mt][t + 2][i], -P.limit), P.limit);
+          v[i] = g * (u + 1.0f) * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * P.alpha * g));
+        }
+      }
+      if (P.vec_store && n + 3 < P.N) {
+        uint2 packed;
+        packed.x = rv_pack_bf16x2(v[0], v[1]);
+        packed.y = rv_pack_bf16x2(v[2], v[3]);
+        *(uint2*)(cr + n) = packed;
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (n + i < P.N) cr[n + i] = rv_f32_to_bf16_bits(v[i]);
+      }
+    }
+  }
+}
+
 // bf16 everywhere.  N: columns of C; with `glu` w holds 2 N rows a group.  groups > 0: the heads' form; 0: the
 // experts' form with tiles of 16 * token_tiles rows.  token_tiles: 1 (few rows) or 4 (many).  K, the leading dimensions of a and w and the group strides of a and w must
 // be multiples of 8 and a, w lie on 16-byte boundaries (a lane reads 16 bytes at a time).
@@ -302,6 +446,14 @@ extern "C" int rv_gemm_groups_mfma(hipStream_t stream, const void* a, const void
   P.a_group_stride = a_group_stride, P.w_group_stride = w_group_stride, P.c_group_stride = c_group_stride;
   P.limit = limit, P.alpha = alpha;
   P.vec_store = (ldc % 4 == 0 && c_group_stride % 4 == 0 && ((uintptr_t)c & 7) == 0) ? 1 : 0;
+  if (groups == 0 && token_tiles == 4 && gate == nullptr) {  // the experts' products of many rows: tiles through LDS
+    dim3 grid(rv_div_up(N, glu ? GL_BW / 2 : GL_BW), rv_div_up(M, GL_BM)), block(256);
+    RV_CHECK(grid.y < 65536, "gemm_groups_mfma: too many row tiles for one launch");
+    if (glu) gemm_experts_lds_kernel<true><<<grid, block, 0, stream>>>(P);
+    else gemm_experts_lds_kernel<false><<<grid, block, 0, stream>>>(P);
+    RV_LAUNCH_CHECK("gemm_experts_lds");
+    return 0;
+  }
   const int rows_of_w = token_tiles == 1 ? 16 : (glu ? 32 : 64);  // of a wave
   dim3 grid(rv_div_up(N, rows_of_w * 4), rv_div_up(M, 16 * token_tiles), groups > 0 ? groups : 1), block(256);
   RV_CHECK(grid.y < 65536 && grid.z < 65536, "gemm_groups_mfma: too many row tiles or groups for one launch");

@@ -222,7 +222,8 @@ def test_products_by_head_with_and_without_a_gate(dtype, rows, heads, n, k):
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("tokens,experts,top,width,inner", [(1, 8, 1, 64, 24), (7, 5, 2, 40, 20), (300, 70, 3, 96, 36),
                                                            (65, 3, 3, 100, 50), (130, 2, 1, 72, 8), (33, 4, 2, 256, 200),
-                                                           (16, 1, 1, 32, 72), (17, 9, 4, 128, 64), (400, 6, 2, 64, 40)])
+                                                           (16, 1, 1, 32, 72), (17, 9, 4, 128, 64), (400, 6, 2, 64, 40),
+                                                           (300, 4, 2, 72, 200), (500, 16, 3, 256, 136), (129, 2, 2, 512, 264)])
 def test_experts_chosen_by_the_tokens_id(dtype, tokens, experts, top, width, inner):
     g = torch.Generator().manual_seed(tokens + experts)
     vocab, limit = 53, 0.8
