@@ -21,7 +21,7 @@ from __future__ import annotations
 import dataclasses
 from typing import Hashable, Optional, Sequence
 
-from ..parts.base import KVNeed, StateNeed
+from ..parts.base import KVNeed, StateNeed, atomic_needs
 from .pages import BlockTable, CacheBookkeepingError, OutOfPages, PagePool, StateSlots
 
 
@@ -106,8 +106,9 @@ class Reservation:
 
 class CacheManager:
     def __init__(self, needs: Sequence, page_size: int, num_pages, max_requests: int):
-        """``needs[i]`` is layer i's need (KVNeed, StateNeed or None).
-        ``num_pages`` is an int (every group gets as many) or a dict by group name."""
+        """``needs[i]`` is layer i's need: KVNeed, StateNeed, None, or a tuple of these for a layer whose mixer
+        holds several (keys in pages beside a state, say).  ``num_pages`` is an int (every group gets as many) or
+        a dict by group name."""
         if page_size < 1:
             raise ValueError("page_size must be positive")
         self.page_size = page_size
@@ -117,17 +118,19 @@ class CacheManager:
         self.layer_group: list[Optional[str]] = []
         self.state_layers: list[int] = []
         for i, need in enumerate(self.needs):
-            if isinstance(need, KVNeed):
-                name = group_name(need.window)
-                if name not in self.groups:
-                    n = num_pages[name] if isinstance(num_pages, dict) else num_pages
-                    self.groups[name] = PageGroup(name, need.window, page_size, int(n))
-                self.groups[name].layers.append(i)
-                self.layer_group.append(name)
-            else:
-                self.layer_group.append(None)
-                if isinstance(need, StateNeed):
+            first_group = None  # of the layer's first need in pages
+            for single in atomic_needs(need):
+                if isinstance(single, KVNeed):
+                    name = group_name(single.window)
+                    if name not in self.groups:
+                        n = num_pages[name] if isinstance(num_pages, dict) else num_pages
+                        self.groups[name] = PageGroup(name, single.window, page_size, int(n))
+                    if i not in self.groups[name].layers:
+                        self.groups[name].layers.append(i)
+                    first_group = first_group or name
+                elif isinstance(single, StateNeed) and i not in self.state_layers:
                     self.state_layers.append(i)
+            self.layer_group.append(first_group)
         self.slots = StateSlots(max_requests)
         self.requests: dict[Hashable, RequestCache] = {}
 

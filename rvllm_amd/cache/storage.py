@@ -22,8 +22,8 @@ import torch
 
 VALUE_GROUP = 16  # slots whose values of one dimension lie side by side (csrc/kv_layout.h)
 
-from ..parts.base import KVCacheView, KVNeed, StateNeed, StateView
-from .manager import CacheManager
+from ..parts.base import KVCacheView, KVNeed, StateNeed, StateView, atomic_needs
+from .manager import CacheManager, group_name
 
 
 class CacheTooLarge(MemoryError):
@@ -34,15 +34,16 @@ def bytes_needed(manager: CacheManager, dtype: torch.dtype) -> int:
     """What ``CacheStorage`` allocates for these books."""
     elem = torch.empty((), dtype=dtype).element_size()
     total = 0
-    for i, need in enumerate(manager.needs):
-        if isinstance(need, KVNeed):
-            g = manager.groups[manager.layer_group[i]]
-            total += 2 * g.pool.num_pages * need.num_kv_heads * g.page_size * need.head_dim * elem
-        elif isinstance(need, StateNeed):
-            count = 1
-            for n in need.shape:
-                count *= int(n)
-            total += manager.max_requests * count * torch.empty((), dtype=need.dtype).element_size()
+    for layer_need in manager.needs:
+        for need in atomic_needs(layer_need):
+            if isinstance(need, KVNeed):
+                g = manager.groups[group_name(need.window)]
+                total += 2 * g.pool.num_pages * need.num_kv_heads * g.page_size * need.head_dim * elem
+            elif isinstance(need, StateNeed):
+                count = 1
+                for n in need.shape:
+                    count *= int(n)
+                total += manager.max_requests * count * torch.empty((), dtype=need.dtype).element_size()
     return total
 
 
@@ -69,26 +70,38 @@ class CacheStorage:
                     f"the cache for {manager.max_requests} requests needs {need_bytes / 2**30:.1f} GiB, "
                     f"{free / 2**30:.1f} GiB of {total / 2**30:.1f} GiB are free{weights}; lower max_cache_tokens, "
                     f"max_num_seqs or max_model_len")
-        for i, need in enumerate(manager.needs):
-            if isinstance(need, KVNeed):
-                g = manager.groups[manager.layer_group[i]]
-                kv = torch.zeros((2, g.pool.num_pages, need.num_kv_heads, g.page_size * need.head_dim), dtype=dtype,
-                                 device=self.device)
-                self.bytes += kv.numel() * kv.element_size()
-                keys = kv[0].view(g.pool.num_pages, need.num_kv_heads, g.page_size, need.head_dim)
-                if g.page_size % VALUE_GROUP:
-                    raise ValueError(f"page_size {g.page_size} must be a multiple of {VALUE_GROUP}: the values are "
-                                     f"transposed by groups of that many slots")
-                values = kv[1].view(g.pool.num_pages, need.num_kv_heads, g.page_size // VALUE_GROUP, need.head_dim,
-                                    VALUE_GROUP)
-                self.views.append(KVCacheView(keys, values, g.name, g.page_size))
-            elif isinstance(need, StateNeed):
-                slots = torch.zeros((manager.max_requests, *need.shape), dtype=need.dtype, device=self.device)
-                self.bytes += slots.numel() * slots.element_size()
-                self.views.append(StateView(slots))
-            else:
-                self.views.append(None)
+        for need in manager.needs:
+            self.views.append(self._view(need))  # a layer whose mixer declares a tuple of needs gets the tuple of views
+
+    def _view(self, need):
+        manager, dtype = self.manager, self.dtype
+        if isinstance(need, KVNeed):
+            g = manager.groups[group_name(need.window)]
+            kv = torch.zeros((2, g.pool.num_pages, need.num_kv_heads, g.page_size * need.head_dim), dtype=dtype,
+                             device=self.device)
+            self.bytes += kv.numel() * kv.element_size()
+            keys = kv[0].view(g.pool.num_pages, need.num_kv_heads, g.page_size, need.head_dim)
+            if g.page_size % VALUE_GROUP:
+                raise ValueError(f"page_size {g.page_size} must be a multiple of {VALUE_GROUP}: the values are "
+                                 f"transposed by groups of that many slots")
+            values = kv[1].view(g.pool.num_pages, need.num_kv_heads, g.page_size // VALUE_GROUP, need.head_dim,
+                                VALUE_GROUP)
+            return KVCacheView(keys, values, g.name, g.page_size)
+        if isinstance(need, StateNeed):
+            slots = torch.zeros((manager.max_requests, *need.shape), dtype=need.dtype, device=self.device)
+            self.bytes += slots.numel() * slots.element_size()
+            return StateView(slots)
+        if isinstance(need, (tuple, list)):
+            return tuple(self._view(member) for member in need)
+        return None
 
     def clear_slot(self, slot: int) -> None:
+        def clear(view):
+            if isinstance(view, StateView):
+                view.slots[slot].zero_()
+            elif isinstance(view, tuple):
+                for member in view:
+                    clear(member)
+
         for i in self.manager.state_layers:
-            self.views[i].slots[slot].zero_()
+            clear(self.views[i])

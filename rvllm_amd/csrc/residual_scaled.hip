@@ -1,0 +1,154 @@
+// The sandwich of norms around a branch with the residual stream kept in 32 bits and a learned scale a channel:
+//
+//   rmsnorm_cast         y = x / sqrt(mean(x^2) + eps) * (offset + w)          x of one type, y of another
+//   add_rmsnorm_scaled   x <- x + branch / sqrt(mean(branch^2) + eps) * (offset + w_post) * scale
+//                        next = x / sqrt(mean(x^2) + eps_next) * (offset_next + w_next)   optionally
+//
+// x is float whatever the activations' type T; the branch is stored as T or given as unreduced 32-bit partial sums
+// of a product; `scale` (one number a channel) may be null.  All arithmetic is 32-bit.  A block takes a row, and
+// the order of a row's additions depends on the width alone.
+#include "common.h"
+
+#define RS_THREADS 256
+
+template <typename TI, typename TO>
+__global__ void __launch_bounds__(RS_THREADS)
+rmsnorm_cast_kernel(const TI* __restrict__ x, const int* __restrict__ row_index, const void* __restrict__ w, int w_f32,
+                    TO* __restrict__ y, int width, float eps, float offset) {
+  __shared__ float scratch[16];
+  const int in_row = row_index ? row_index[blockIdx.x] : (int)blockIdx.x;
+  const TI* xr = x + (size_t)in_row * width;
+  TO* yr = y + (size_t)blockIdx.x * width;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < width; i += RS_THREADS) {
+    const float v = rv_to_float(xr[i]);
+    ss = fmaf(v, v, ss);
+  }
+  ss = rv_block_sum(ss, scratch);
+  const float inv = 1.0f / sqrtf(ss / (float)width + eps);
+  for (int i = threadIdx.x; i < width; i += RS_THREADS)
+    yr[i] = rv_from_float<TO>(rv_to_float(xr[i]) * inv * (offset + rv_load_w(w, w_f32, i)));
+}
+
+extern "C" int rv_rmsnorm_cast(hipStream_t stream, const void* x, int x_dtype, const int* row_index, const void* w,
+                               int w_f32, void* y, int y_dtype, int rows, int width, float eps, float offset) {
+  RV_CHECK(rows >= 0 && width > 0 && x && w && y, "rmsnorm_cast: bad arguments rows=%d width=%d", rows, width);
+  if (rows == 0) return 0;
+  dim3 grid(rows), block(RS_THREADS);
+#define RV_NC(TI, TO) \
+  rmsnorm_cast_kernel<TI, TO><<<grid, block, 0, stream>>>((const TI*)x, row_index, w, w_f32, (TO*)y, width, eps, offset)
+  if (x_dtype == RV_F32 && y_dtype == RV_F32) RV_NC(float, float);
+  else if (x_dtype == RV_F32 && y_dtype == RV_BF16) RV_NC(float, bf16_t);
+  else if (x_dtype == RV_BF16 && y_dtype == RV_BF16) RV_NC(bf16_t, bf16_t);
+  else return rv_fail("rmsnorm_cast: unsupported dtypes %d -> %d", x_dtype, y_dtype);
+#undef RV_NC
+  RV_LAUNCH_CHECK("rmsnorm_cast");
+  return 0;
+}
+
+template <typename T>
+__device__ __forceinline__ float rs_branch(const void* p, int slices, long long stride, size_t at) {
+  if (slices == 0) return rv_to_float(((const T*)p)[at]);
+  float v = 0.f;
+  for (int s = 0; s < slices; ++s) v += ((const float*)p)[(size_t)s * stride + at];
+  return v;
+}
+
+template <typename T>
+__global__ void __launch_bounds__(RS_THREADS)
+add_rmsnorm_scaled_kernel(const void* __restrict__ branch, int slices, long long slice_stride,
+                          const void* __restrict__ w_post, int w_post_f32, const void* __restrict__ scale,
+                          int scale_f32, float* __restrict__ x, const void* __restrict__ w_next, int w_next_f32,
+                          T* __restrict__ next, int width, float eps, float offset, float eps_next,
+                          float offset_next) {
+  __shared__ float scratch[16];
+  const size_t row0 = (size_t)blockIdx.x * width;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < width; i += RS_THREADS) {
+    const float v = rs_branch<T>(branch, slices, slice_stride, row0 + i);
+    ss = fmaf(v, v, ss);
+  }
+  ss = rv_block_sum(ss, scratch);
+  const float inv = 1.0f / sqrtf(ss / (float)width + eps);
+  float ss2 = 0.f;
+  for (int i = threadIdx.x; i < width; i += RS_THREADS) {
+    float v = rs_branch<T>(branch, slices, slice_stride, row0 + i) * inv * (offset + rv_load_w(w_post, w_post_f32, i));
+    if (scale) v *= rv_load_w(scale, scale_f32, i);
+    const float r = x[row0 + i] + v;
+    x[row0 + i] = r;
+    ss2 = fmaf(r, r, ss2);
+  }
+  if (next == nullptr) return;
+  ss2 = rv_block_sum(ss2, scratch);
+  const float inv2 = 1.0f / sqrtf(ss2 / (float)width + eps_next);
+  // every thread reads back what it wrote itself
+  for (int i = threadIdx.x; i < width; i += RS_THREADS)
+    next[row0 + i] = rv_from_float<T>(x[row0 + i] * inv2 * (offset_next + rv_load_w(w_next, w_next_f32, i)));
+}
+
+// branch: `dtype` values [rows, width] (slices 0) or 32-bit partial sums [slices][rows][width]; x: float, in place;
+// next: `dtype`, with w_next, or both null.
+extern "C" int rv_add_rmsnorm_scaled(hipStream_t stream, const void* branch, int slices, long long slice_stride,
+                                     const void* w_post, int w_post_f32, const void* scale, int scale_f32, float* x,
+                                     const void* w_next, int w_next_f32, void* next, int dtype, int rows, int width,
+                                     float eps, float offset, float eps_next, float offset_next) {
+  RV_CHECK(rows >= 0 && width > 0 && branch && w_post && x, "add_rmsnorm_scaled: bad arguments rows=%d width=%d", rows,
+           width);
+  RV_CHECK((w_next == nullptr) == (next == nullptr), "add_rmsnorm_scaled: the next norm needs both weight and output");
+  RV_CHECK(slices >= 0 && (slices == 0 || slice_stride >= (long long)rows * width), "add_rmsnorm_scaled: bad partial sums");
+  if (rows == 0) return 0;
+  dim3 grid(rows), block(RS_THREADS);
+#define RV_AS(T)                                                                                                      \
+  add_rmsnorm_scaled_kernel<T><<<grid, block, 0, stream>>>(branch, slices, slice_stride, w_post, w_post_f32, scale,   \
+                                                           scale_f32, x, w_next, w_next_f32, (T*)next, width, eps,    \
+                                                           offset, eps_next, offset_next)
+  if (dtype == RV_F32) RV_AS(float);
+  else if (dtype == RV_BF16) RV_AS(bf16_t);
+  else return rv_fail("add_rmsnorm_scaled: unsupported dtype %d", dtype);
+#undef RV_AS
+  RV_LAUNCH_CHECK("add_rmsnorm_scaled");
+  return 0;
+}
+
+// x[i] = x[i] * a over `total` 32-bit numbers (the logits' multiplier).
+__global__ void scale_f32_kernel(float* __restrict__ x, long long total, float a) {
+  const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx < total) x[idx] *= a;
+}
+
+extern "C" int rv_scale_f32(hipStream_t stream, float* x, long long total, float a) {
+  RV_CHECK(total >= 0 && x, "scale_f32: bad arguments");
+  if (total == 0) return 0;
+  scale_f32_kernel<<<dim3(rv_div_up(total, 256)), dim3(256), 0, stream>>>(x, total, a);
+  RV_LAUNCH_CHECK("scale_f32");
+  return 0;
+}
+
+// out[t][c] = a * x[t][c] + b * y[t][c]: two mixers side by side, each with its weight; x and y of type `dtype` or
+// unreduced 32-bit partial sums of a product; the sum is 32-bit and stays 32-bit (the consumer takes it as the one
+// slice of a product's partial sums).
+template <typename T>
+__global__ void weighted_sum_kernel(const void* __restrict__ x, int x_slices, long long x_stride,
+                                    const void* __restrict__ y, int y_slices, long long y_stride, float a, float b,
+                                    float* __restrict__ out, long long total) {
+  const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= total) return;
+  out[idx] = a * rs_branch<T>(x, x_slices, x_stride, (size_t)idx) + b * rs_branch<T>(y, y_slices, y_stride, (size_t)idx);
+}
+
+extern "C" int rv_weighted_sum(hipStream_t stream, const void* x, int x_slices, long long x_stride, const void* y,
+                               int y_slices, long long y_stride, float a, float b, float* out, int dtype, int rows,
+                               int width) {
+  RV_CHECK(x && y && out && rows >= 0 && width > 0, "weighted_sum: bad arguments");
+  if (rows == 0) return 0;
+  const long long total = (long long)rows * width;
+  dim3 grid(rv_div_up(total, 256)), block(256);
+  if (dtype == RV_F32)
+    weighted_sum_kernel<float><<<grid, block, 0, stream>>>(x, x_slices, x_stride, y, y_slices, y_stride, a, b, out, total);
+  else if (dtype == RV_BF16)
+    weighted_sum_kernel<bf16_t><<<grid, block, 0, stream>>>(x, x_slices, x_stride, y, y_slices, y_stride, a, b, out, total);
+  else
+    return rv_fail("weighted_sum: unsupported dtype %d", dtype);
+  RV_LAUNCH_CHECK("weighted_sum");
+  return 0;
+}

@@ -25,7 +25,7 @@ from ..config.engine_config import EngineConfig
 from ..kernels import ops
 from ..models.model import DecoderModel
 from ..models.registry import Architecture, get_architecture, load_config
-from ..parts.base import KVNeed
+from ..parts.base import KVNeed, atomic_needs
 from ..weights.loader import load_tensors, open_model_files, tensor_names
 from ..weights.random_init import random_tensors
 from .batch import BatchBuilder, Portion, StepBatch
@@ -63,7 +63,8 @@ class ModelRunner:
         needs = model.cache_needs()
         full_pages = max(1, -(-cfg.cache_tokens() // ps))
         num_pages = {}
-        for need in needs:
+        singles = [single for need in needs for single in atomic_needs(need)]
+        for need in singles:
             if isinstance(need, KVNeed):
                 name = group_name(need.window)
                 if need.window is None:
@@ -85,7 +86,7 @@ class ModelRunner:
         # but keys and values between steps (replaying such a step writes the same keys and values again, so the
         # check below may replay it; a state that a mixer moves on would be moved on with every replay), and
         # until a recording fails its check.
-        self._library_steps_from_graphs = all(need is None or isinstance(need, KVNeed) for need in needs)
+        self._library_steps_from_graphs = all(isinstance(need, KVNeed) for need in singles)
         _freeze_what_exists_once()
 
     # ---- decode steps from captured graphs -------------------------------

@@ -1372,3 +1372,275 @@ def gemm_bf16_gate_up(x: torch.Tensor, w_fours, activation: str):
                                       _c_ll(0 if tiled else (w_fours.stride(0) if n > 1 else k)), _c_ll(n // 2),
                                       _c_int(ACTIVATIONS[activation]), _c_int(int(tiled))))
     return out
+
+
+# ---- a 32-bit residual stream between sandwiched branches ---------------------------------------------------
+def rmsnorm_cast(x: torch.Tensor, weight: torch.Tensor, eps: float, offset: float, out_dtype: torch.dtype,
+                 out: Optional[torch.Tensor] = None, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Row-wise RMSNorm whose result has another type than its input (a 32-bit residual stream, activations in
+    bf16).  ``rows`` as in ``rmsnorm``."""
+    _gpu(x, weight, out, rows)
+    _need(x.dim() == 2, "rmsnorm_cast: a matrix is expected")
+    width = x.shape[1]
+    _need(weight.shape == (width,) and weight.dtype in _DT, f"rmsnorm_cast: the weight must hold {width} numbers")
+    if rows is not None:
+        _i32(rows)
+    n_rows = x.shape[0] if rows is None else rows.numel()
+    if out is None:
+        out = torch.empty((n_rows, width), dtype=out_dtype, device=x.device)
+    _need(out.shape == (n_rows, width) and out.dtype == out_dtype, "rmsnorm_cast: bad out")
+    _check(library().rv_rmsnorm_cast(_stream(), _ptr(x), _dt(x), _ptr(rows), _ptr(weight),
+                                     _c_int(weight.dtype == torch.float32), _ptr(out), _dt(out), _c_int(n_rows),
+                                     _c_int(width), _c_float(eps), _c_float(offset)))
+    return out
+
+
+def add_rmsnorm_scaled(branch, weight: torch.Tensor, eps: float, offset: float, scale: Optional[torch.Tensor],
+                       residual: torch.Tensor, next_weight: Optional[torch.Tensor] = None, next_eps: float = 0.0,
+                       next_offset: float = 0.0) -> Optional[torch.Tensor]:
+    """residual += rmsnorm(branch) * scale on a 32-bit ``residual``; ``scale`` is one number a channel or None.
+    With ``next_weight`` also returns rmsnorm(residual) in the branch's type.  ``branch`` is a tensor of the
+    activations' type or ``SlicedSums``."""
+    bptr, slices, stride, rows, width, bdtype = _branch_args(branch, "add_rmsnorm_scaled")
+    _gpu(weight, scale, residual, next_weight)
+    _need(residual.shape == (rows, width) and residual.dtype == torch.float32,
+          "add_rmsnorm_scaled: the residual stream is a 32-bit matrix of the branch's shape")
+    _need(weight.shape == (width,) and weight.dtype in _DT, "add_rmsnorm_scaled: bad weight")
+    _need(scale is None or (scale.shape == (width,) and scale.dtype in _DT), "add_rmsnorm_scaled: bad scale")
+    nxt = None
+    if next_weight is not None:
+        _need(next_weight.shape == (width,) and next_weight.dtype in _DT, "add_rmsnorm_scaled: bad next weight")
+        nxt = torch.empty((rows, width), dtype=bdtype, device=residual.device)
+    _check(library().rv_add_rmsnorm_scaled(
+        _stream(), bptr, _c_int(slices), _c_ll(stride), _ptr(weight), _c_int(weight.dtype == torch.float32),
+        _ptr(scale), _c_int(scale is not None and scale.dtype == torch.float32), _ptr(residual), _ptr(next_weight),
+        _c_int(next_weight is not None and next_weight.dtype == torch.float32), _ptr(nxt), _DT[bdtype], _c_int(rows),
+        _c_int(width), _c_float(eps), _c_float(offset), _c_float(next_eps), _c_float(next_offset)))
+    return nxt
+
+
+def scale_(x: torch.Tensor, a: float) -> torch.Tensor:
+    """x *= a for a 32-bit tensor, in place."""
+    _gpu(x)
+    _need(x.dtype == torch.float32, "scale_: a 32-bit tensor expected")
+    _check(library().rv_scale_f32(_stream(), _ptr(x), _c_ll(x.numel()), _c_float(a)))
+    return x
+
+
+def weighted_sum(x, y, a: float, b: float) -> SlicedSums:
+    """a * x + b * y for two branches (tensors of one type or unreduced ``SlicedSums``), added in 32-bit and left
+    32-bit: the result is handed on as the one slice of a product's partial sums."""
+    xptr, x_slices, x_stride, rows, width, dtype = _branch_args(x, "weighted_sum")
+    yptr, y_slices, y_stride, y_rows, y_width, y_dtype = _branch_args(y, "weighted_sum")
+    _need((rows, width, dtype) == (y_rows, y_width, y_dtype), "weighted_sum: two branches of one shape and type")
+    out = torch.empty((1, rows, width), dtype=torch.float32, device=x.device)
+    _check(library().rv_weighted_sum(_stream(), xptr, _c_int(x_slices), _c_ll(x_stride), yptr, _c_int(y_slices),
+                                     _c_ll(y_stride), _c_float(a), _c_float(b), _ptr(out), _DT[dtype], _c_int(rows),
+                                     _c_int(width)))
+    return SlicedSums(out, dtype)
+
+
+# ---- attention with a partial rotation in halves, a norm after it, values that are the keys ----------------------
+NORM_NONE, NORM_BEFORE_ROTATION, NORM_AFTER_ROTATION = 0, 1, 2
+
+
+def rotate_norm_write(proj: torch.Tensor, q_col: int, k_col: int, v_col: Optional[int], q_out: torch.Tensor,
+                      q_weight: Optional[torch.Tensor], k_weight: Optional[torch.Tensor], eps: float, offset: float,
+                      norm_mode: int, rope: Optional[tuple[torch.Tensor, torch.Tensor]], rotary_dim: int,
+                      positions: torch.Tensor, token_req: torch.Tensor, block_table: Optional[torch.Tensor],
+                      k_pages: Optional[torch.Tensor], v_pages: Optional[torch.Tensor], num_q_heads: int,
+                      num_kv_heads: int, head_dim: int, write_kv: bool = True) -> torch.Tensor:
+    """Queries and keys from the rows of ``proj`` (queries from column ``q_col``, keys from ``k_col``, values from
+    ``v_col`` or, with None, the keys as they stand there): rotation of the first ``rotary_dim`` dimensions of a
+    head, dimension i paired with i + rotary_dim / 2; per-head RMS norm before or after it (``norm_mode``), with
+    the weights or without; queries to ``q_out``, keys and values into the cache."""
+    cos, sin = rope if rope is not None else (None, None)
+    _gpu(q_out, q_weight, k_weight, cos, sin, positions, token_req, block_table, k_pages, v_pages)
+    _need(proj.is_cuda and proj.dim() == 2 and proj.stride(1) == 1, "rotate_norm_write: rows of projections expected")
+    _i32(positions, token_req)
+    n = proj.shape[0]
+    q_size, kv_size = num_q_heads * head_dim, num_kv_heads * head_dim
+    cols = proj.shape[1]
+    _need(0 <= q_col and q_col + q_size <= cols and 0 <= k_col and k_col + kv_size <= cols
+          and (v_col is None or (0 <= v_col and v_col + kv_size <= cols)), "rotate_norm_write: columns outside the rows")
+    _need(q_out.shape == (n, q_size) and q_out.dtype == proj.dtype, "rotate_norm_write: bad q_out")
+    _need(positions.numel() >= n and token_req.numel() >= n, "rotate_norm_write: positions/token_req too short")
+    w_f32 = 0
+    if q_weight is not None or k_weight is not None:
+        _need(q_weight is not None and k_weight is not None and q_weight.shape == (head_dim,)
+              and k_weight.shape == (head_dim,) and q_weight.dtype == k_weight.dtype and q_weight.dtype in _DT,
+              "rotate_norm_write: bad norm weights")
+        w_f32 = int(q_weight.dtype == torch.float32)
+    rot = rotary_dim if rope is not None else 0
+    if rot:
+        for table in (cos, sin):
+            _need(table.dtype == torch.float32 and table.shape == (n, rot // 2),
+                  f"rotate_norm_write: the table of cosines and sines must be 32-bit [{n}, {rot // 2}]")
+    page_size = num_pages = width = 0
+    if write_kv:
+        _need(k_pages is not None and v_pages is not None and block_table is not None, "rotate_norm_write: no cache given")
+        _i32(block_table)
+        num_pages, nkv, page_size, hd = _cache_geometry(k_pages, v_pages, "rotate_norm_write")
+        _need((nkv, hd) == (num_kv_heads, head_dim), "rotate_norm_write: cache pages do not fit the heads")
+        _need(k_pages.dtype == proj.dtype and v_pages.dtype == proj.dtype, "rotate_norm_write: cache dtype differs")
+        width = block_table.shape[1]
+    _check(library().rv_rotate_norm_write(
+        _stream(), _ptr(proj), _c_ll(proj.stride(0)), _c_int(q_col), _c_int(k_col), _c_int(-1 if v_col is None else v_col),
+        _ptr(q_out), _ptr(q_weight), _ptr(k_weight), _c_int(w_f32), _c_float(eps), _c_float(offset), _c_int(norm_mode),
+        _ptr(cos), _ptr(sin), _c_int(rot), _ptr(positions), _ptr(token_req), _ptr(block_table), _c_int(width),
+        _ptr(k_pages), _ptr(v_pages), _c_int(page_size), _c_int(num_pages), _dt(proj), _c_int(n), _c_int(num_q_heads),
+        _c_int(num_kv_heads), _c_int(head_dim), _c_int(int(write_kv))))
+    return q_out
+
+
+GATE_ACTS = {"sigmoid": 0, "silu": 1}
+
+
+def gate_mul_(a: torch.Tensor, gate: torch.Tensor, gate_col0: int, act: str) -> torch.Tensor:
+    """a[t, c] *= act(gate[t, gate_col0 + c]), in place; ``act`` is ``sigmoid`` or ``silu``."""
+    _gpu(a)
+    _need(gate.is_cuda and gate.dim() == 2 and gate.stride(1) == 1 and a.dim() == 2 and gate.dtype == a.dtype
+          and gate.shape[0] == a.shape[0] and 0 <= gate_col0 and gate_col0 + a.shape[1] <= gate.shape[1],
+          "gate_mul: the gate must hold the columns of a in its rows")
+    _need(act in GATE_ACTS, f"gate_mul: unknown activation {act!r}")
+    _check(library().rv_gate_mul(_stream(), _ptr(a), gate.data_ptr() + gate_col0 * gate.element_size(),
+                                 _c_ll(gate.stride(0)), _dt(a), _c_int(a.shape[0]), _c_int(a.shape[1]),
+                                 _c_int(GATE_ACTS[act])))
+    return a
+
+
+# ---- mixers with a state of fixed size ------------------------------------------------------------------------
+def _state_args(slots: torch.Tensor, what: str) -> int:
+    _gpu(slots)
+    _need(slots.dim() == 2 and slots.dtype == torch.float32, f"{what}: the state slots are 32-bit [slots, size]")
+    return slots.stride(0)
+
+
+def causal_conv(x: torch.Tensor, col0: int, channels: int, weight: torch.Tensor, bias: Optional[torch.Tensor],
+                slots: torch.Tensor, state_off: int, step, out: torch.Tensor, out_col0: int = 0, group: int = 64,
+                unit_eps: Optional[float] = None, scaled_groups: int = 0, group_scale: float = 1.0,
+                state_ld: Optional[int] = None) -> torch.Tensor:
+    """Short causal convolution over time and silu for the channels ``col0 .. col0 + channels`` of the rows of
+    ``x``: ``weight`` is float32 ``[channels, taps]`` (the last tap is the token's own), ``bias`` float32 or None.
+    The inputs before a request's first token of the step come from its state slot (``taps - 1`` rows of
+    ``channels`` floats from ``state_off`` on), which this call only reads (``conv_state_update`` moves it on).
+    Results go to the columns ``out_col0 ...`` of ``out`` (float32 or the type of ``x``).  With ``unit_eps`` every
+    group of ``group`` channels is divided by sqrt(sum of squares + unit_eps), and the first ``scaled_groups``
+    groups are multiplied by ``group_scale``.  ``state_ld``: the channels a row of the state holds, when these
+    are a part of them (``state_off`` then points at this part's first channel)."""
+    _gpu(weight, bias)
+    state_ld = channels if state_ld is None else int(state_ld)
+    _need(x.is_cuda and x.dim() == 2 and x.stride(1) == 1 and out.is_cuda and out.dim() == 2 and out.stride(1) == 1,
+          "causal_conv: rows expected")
+    n = x.shape[0]
+    _need(n == step.num_tokens and out.shape[0] == n, "causal_conv: the rows must be the step's tokens")
+    _need(0 <= col0 and col0 + channels <= x.shape[1] and 0 <= out_col0 and out_col0 + channels <= out.shape[1],
+          "causal_conv: channels outside the rows")
+    _need(weight.dim() == 2 and weight.shape[0] == channels and weight.dtype == torch.float32
+          and (bias is None or (bias.shape == (channels,) and bias.dtype == torch.float32)),
+          "causal_conv: float32 weights [channels, taps] and bias [channels] expected")
+    _need(out.dtype == torch.float32 or out.dtype == x.dtype, "causal_conv: the result is float32 or of the input's type")
+    taps = weight.shape[1]
+    stride = _state_args(slots, "causal_conv")
+    _need(state_ld >= channels and 0 <= state_off
+          and state_off + max(0, taps - 2) * state_ld + (channels if taps > 1 else 0) <= slots.shape[1],
+          "causal_conv: the state lies outside the slot")
+    _check(library().rv_causal_conv(
+        _stream(), x.data_ptr() + col0 * x.element_size(), _dt(x), _c_ll(x.stride(0)), _ptr(weight), _ptr(bias),
+        _c_int(taps), _ptr(slots), _c_ll(stride), _c_ll(state_off), _c_int(state_ld), _ptr(step.positions),
+        _ptr(step.token_req), _ptr(step.q_start), _ptr(step.chunk_start), _ptr(step.state_slot),
+        out.data_ptr() + out_col0 * out.element_size(), _c_int(out.dtype == torch.float32 and x.dtype != torch.float32),
+        _c_ll(out.stride(0)), _c_int(channels), _c_int(group), _c_int(n),
+        _c_float(-1.0 if unit_eps is None else unit_eps), _c_int(scaled_groups), _c_float(group_scale)))
+    return out
+
+
+def conv_state_update(x: torch.Tensor, col0: int, channels: int, taps: int, slots: torch.Tensor, state_off: int,
+                      step) -> None:
+    """The convolution's state of every request of the step becomes the last ``taps - 1`` inputs it has seen."""
+    _need(x.is_cuda and x.dim() == 2 and x.stride(1) == 1 and 0 <= col0 and col0 + channels <= x.shape[1],
+          "conv_state_update: channels outside the rows")
+    stride = _state_args(slots, "conv_state_update")
+    _need(0 <= state_off and state_off + (taps - 1) * channels <= slots.shape[1],
+          "conv_state_update: the state lies outside the slot")
+    _check(library().rv_conv_state_update(
+        _stream(), x.data_ptr() + col0 * x.element_size(), _dt(x), _c_ll(x.stride(0)), _c_int(taps), _ptr(slots),
+        _c_ll(stride), _c_ll(state_off), _c_int(channels), _ptr(step.q_start), _ptr(step.state_slot), _c_int(channels),
+        _c_int(step.num_requests)))
+
+
+def delta_rule(qkv: torch.Tensor, q_off: int, k_off: int, v_off: int, ab: torch.Tensor, a_col: int, b_col: int,
+               A_log: torch.Tensor, dt_bias: torch.Tensor, slots: torch.Tensor, state_off: int, step, heads: int,
+               kv_heads: int, dk: int, dv: int) -> torch.Tensor:
+    """The gated delta rule over the step's tokens, request by request in order.  ``qkv`` float32 rows: unit
+    queries (scaled) and keys of ``kv_heads`` heads of ``dk``, values of ``heads`` heads of ``dv``, at their
+    offsets; ``ab`` rows hold the decay's input of head h at ``a_col + h`` and beta's at ``b_col + h``;
+    g = exp(-exp(A_log) softplus(a + dt_bias)), beta = sigmoid(b).  Per head S [dk, dv] (32-bit, in the
+    request's slot from ``state_off``): S <- g S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q.  Returns o as
+    float32 ``[tokens, heads * dv]``."""
+    _gpu(qkv, A_log, dt_bias)
+    n = qkv.shape[0]
+    _need(qkv.dtype == torch.float32 and qkv.dim() == 2 and n == step.num_tokens, "delta_rule: float32 rows of the step's tokens")
+    _need(ab.is_cuda and ab.dim() == 2 and ab.stride(1) == 1 and ab.shape[0] == n and ab.dtype in _DT
+          and 0 <= a_col and a_col + heads <= ab.shape[1] and 0 <= b_col and b_col + heads <= ab.shape[1],
+          "delta_rule: the gates' inputs lie outside their rows")
+    _need(heads % kv_heads == 0 and max(q_off, k_off) + kv_heads * dk <= qkv.shape[1] and v_off + heads * dv <= qkv.shape[1],
+          "delta_rule: heads outside the rows")
+    _need(A_log.shape == (heads,) and dt_bias.shape == (heads,) and A_log.dtype == torch.float32
+          and dt_bias.dtype == torch.float32, "delta_rule: float32 A_log and dt_bias, one a head")
+    stride = _state_args(slots, "delta_rule")
+    _need(0 <= state_off and state_off + heads * dk * dv <= slots.shape[1], "delta_rule: the state lies outside the slot")
+    out = torch.empty((n, heads * dv), dtype=torch.float32, device=qkv.device)
+    _check(library().rv_delta_rule(
+        _stream(), _ptr(qkv), _c_ll(qkv.stride(0)), _c_int(q_off), _c_int(k_off), _c_int(v_off), _ptr(ab), _dt(ab),
+        _c_ll(ab.stride(0)), _c_int(a_col), _c_int(b_col), _ptr(A_log), _ptr(dt_bias), _ptr(slots), _c_ll(stride),
+        _c_ll(state_off), _ptr(step.q_start), _ptr(step.state_slot), _ptr(out), _c_int(step.num_requests), _c_int(heads),
+        _c_int(kv_heads), _c_int(dk), _c_int(dv)))
+    return out
+
+
+def head_norm_gate(o: torch.Tensor, gate: torch.Tensor, gate_col0: int, weight: torch.Tensor, eps: float, heads: int,
+                   dv: int, out_dtype: torch.dtype) -> torch.Tensor:
+    """out[t, h] = o[t, h] / rms(o[t, h]) * weight * silu(gate[t, gate_col0 + h dv ...]) for every head."""
+    _gpu(o, weight)
+    n = o.shape[0]
+    _need(o.dtype == torch.float32 and o.shape == (n, heads * dv), "head_norm_gate: float32 [tokens, heads * dv]")
+    _need(weight.shape == (dv,) and weight.dtype == torch.float32, "head_norm_gate: a float32 weight of the head's size")
+    _need(gate.is_cuda and gate.dim() == 2 and gate.stride(1) == 1 and gate.dtype == out_dtype and gate.shape[0] == n
+          and 0 <= gate_col0 and gate_col0 + heads * dv <= gate.shape[1], "head_norm_gate: the gate lies outside its rows")
+    out = torch.empty((n, heads * dv), dtype=out_dtype, device=o.device)
+    _check(library().rv_head_norm_gate(_stream(), _ptr(o), gate.data_ptr() + gate_col0 * gate.element_size(),
+                                       _c_ll(gate.stride(0)), _ptr(weight), _ptr(out), _dt(out), _c_int(n), _c_int(heads),
+                                       _c_int(dv), _c_float(eps)))
+    return out
+
+
+def selective_scan(x: torch.Tensor, z: torch.Tensor, z_col0: int, dt: torch.Tensor, dt_bias: torch.Tensor,
+                   bc: torch.Tensor, b_col: int, c_col: int, A_log: torch.Tensor, D: torch.Tensor, slots: torch.Tensor,
+                   state_off: int, step) -> torch.Tensor:
+    """The selective scan over the step's tokens, request by request in order.  ``x [tokens, channels]`` the
+    convolved input, ``z`` the gate's input at ``z_col0`` of its rows, ``dt [tokens, channels]`` the step's
+    projection (step = softplus(dt + dt_bias)), ``bc`` rows with B at ``b_col`` and C at ``c_col`` (``n`` each),
+    A = -exp(A_log [channels, n]), D [channels].  S [channels, n] (32-bit, in the request's slot from
+    ``state_off``): S <- exp(step A) S + step x B; y = S . C + D x.  Returns y * silu(z) in the type of ``x``."""
+    _gpu(x, dt, dt_bias, A_log, D)
+    n, channels = x.shape
+    n_state = A_log.shape[1]
+    _need(n == step.num_tokens and x.dtype in _DT, "selective_scan: the rows must be the step's tokens")
+    _need(dt.shape == (n, channels) and dt.dtype == x.dtype, "selective_scan: bad dt")
+    _need(z.is_cuda and z.dim() == 2 and z.stride(1) == 1 and z.dtype == x.dtype and z.shape[0] == n
+          and 0 <= z_col0 and z_col0 + channels <= z.shape[1], "selective_scan: the gate lies outside its rows")
+    _need(bc.is_cuda and bc.dim() == 2 and bc.stride(1) == 1 and bc.dtype == x.dtype and bc.shape[0] == n
+          and 0 <= b_col and b_col + n_state <= bc.shape[1] and 0 <= c_col and c_col + n_state <= bc.shape[1],
+          "selective_scan: B and C lie outside their rows")
+    _need(A_log.shape == (channels, n_state) and D.shape == (channels,) and dt_bias.shape == (channels,)
+          and A_log.dtype == D.dtype == dt_bias.dtype == torch.float32, "selective_scan: float32 A_log, D and dt_bias")
+    stride = _state_args(slots, "selective_scan")
+    _need(0 <= state_off and state_off + channels * n_state <= slots.shape[1], "selective_scan: the state lies outside the slot")
+    out = torch.empty_like(x)
+    _check(library().rv_selective_scan(
+        _stream(), _ptr(x), _c_ll(x.stride(0)), z.data_ptr() + z_col0 * z.element_size(), _c_ll(z.stride(0)), _ptr(dt),
+        _c_ll(dt.stride(0)), _ptr(dt_bias), _ptr(bc), _c_ll(bc.stride(0)), _c_int(b_col), _c_int(c_col), _ptr(A_log),
+        _ptr(D), _ptr(slots), _c_ll(stride), _c_ll(state_off), _ptr(step.q_start), _ptr(step.state_slot), _ptr(out),
+        _dt(x), _c_int(step.num_requests), _c_int(channels), _c_int(n_state)))
+    return out

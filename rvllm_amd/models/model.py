@@ -13,7 +13,7 @@ from typing import Optional
 import torch
 
 from ..parts import embedding as _embedding  # noqa: F401  (registers the embedding and the head)
-from ..parts.base import ParamSpec
+from ..parts.base import ParamSpec, reader_view
 from ..parts.registry import BLOCKS, EMBEDDINGS, HEADS, NORMS
 from ..parts.spec import ModelSpec
 
@@ -112,7 +112,7 @@ class DecoderModel:
         entered = None
         for i, entry in enumerate(schedule):
             block = self.blocks[entry.layer]
-            cache = caches[entry.layer] if entry.cache_from is None else caches[entry.cache_from].reader()
+            cache = caches[entry.layer] if entry.cache_from is None else reader_view(caches[entry.cache_from])
             nxt = self.blocks[schedule[i + 1].layer].entry_norm() if i + 1 < len(schedule) else None
             # None means the block did not apply the next entry norm; the next block then does
             entered = block.forward(x, step, cache, entered=entered, then=nxt)

@@ -13,6 +13,17 @@ role (``q``, ``k``, ``v``, ``o``, ``q_norm``, ``k_norm``) to the tensor's name u
 the layer's prefix, without ``.weight`` (the Gemma names if absent); a role ``qkv``
 names one stored matrix that holds the rows of q, k and v in this order.  ``bias``
 lists the projections that have a ``.bias`` beside their ``.weight`` (True: all).
+``weight_suffix`` / ``bias_suffix`` are what a projection's name is followed by
+(``.weight`` / ``.bias`` if absent).
+
+Variants, all parameters: ``values`` = ``"keys"``: there is no value projection, a
+token's values are its keys as projected, before norm and rotation.  ``gate`` =
+``"sigmoid"``: the concatenated heads are multiplied by sigmoid of one more
+projection of the layer's input (role ``g``) before the output projection.
+``qk_norm`` may say ``"weight": False`` (a norm without a learned weight) and
+``"after_rotation": True`` (rotate first, then norm).  A position encoding may pair
+dimension i with i + rotary_dim/2 (``rope``'s ``pairing``).  Any of these takes the
+step through ``ops.rotate_norm_write`` instead of the fused kernel of the plain case.
 """
 
 from __future__ import annotations
@@ -48,21 +59,51 @@ class PagedAttention(Mixer):
         self.q_size = self.num_heads * self.head_dim
         self.kv_size = self.num_kv_heads * self.head_dim
         self.names = tensor_names(self.NAMES, spec.get("names"))
+        self.w_suffix = str(spec.get("weight_suffix", ".weight"))
+        self.b_suffix = str(spec.get("bias_suffix", ".bias"))
+        values = str(spec.get("values", "projected"))
+        if values not in ("projected", "keys"):
+            raise ValueError(f"attention: values {values!r}; known: 'projected', 'keys'")
+        self.values_from_keys = values == "keys"
+        gate = spec.get("gate")
+        if gate not in (None, "sigmoid"):
+            raise ValueError(f"attention: gate {gate!r}; known: None, 'sigmoid'")
+        self.gate = gate
+        self.norm_weight = bool((self.qk_norm or {}).get("weight", True))
+        self.norm_after_rotation = bool((self.qk_norm or {}).get("after_rotation", False))
         # the projections as the checkpoint stores them: role -> rows
-        self.stored = ({"qkv": self.q_size + 2 * self.kv_size} if "qkv" in self.names
-                       else {"q": self.q_size, "k": self.kv_size, "v": self.kv_size})
+        if "qkv" in self.names:
+            if self.values_from_keys or self.gate:
+                raise ValueError("attention: a stored q|k|v matrix goes with projected values and no gate")
+            self.stored = {"qkv": self.q_size + 2 * self.kv_size}
+        else:
+            self.stored = {"q": self.q_size, "k": self.kv_size}
+            if not self.values_from_keys:
+                self.stored["v"] = self.kv_size
+            if self.gate:
+                self.names.setdefault("g", "self_attn.g_proj")
+                self.stored["g"] = self.q_size
         self.bias = bias_roles(spec.get("bias"), [*self.stored, "o"])
+        # the step's kernel for queries and keys: the fused one of the plain case, or the general one
+        partial_halves = (self.position.rotary_dim not in (0, self.head_dim)
+                          and getattr(self.position, "pairing", "head_half") == "rotary_half")
+        self.general_path = bool(self.values_from_keys or self.gate or partial_halves or self.norm_after_rotation
+                                 or (self.qk_norm is not None and not self.norm_weight))
+        if self.general_path and self.position.rotary_dim not in (0, self.head_dim) \
+                and getattr(self.position, "pairing", "head_half") != "rotary_half":
+            raise ValueError("attention: with these variants a partial rotation pairs i with i + rotary_dim/2")
         self.w_qkv = self.w_o = self.q_norm_w = self.k_norm_w = self.b_qkv = self.b_o = None
 
     # ---- weights -----------------------------------------------------
     def param_specs(self, prefix: str) -> list[ParamSpec]:
         at = {role: f"{prefix}.{name}" for role, name in self.names.items()}
-        specs = [ParamSpec(f"{at[role]}.weight", (rows, self.hidden_size)) for role, rows in self.stored.items()]
-        specs.append(ParamSpec(f"{at['o']}.weight", (self.hidden_size, self.q_size)))
-        specs += [ParamSpec(f"{at[role]}.bias", (rows,)) for role, rows in self.stored.items() if role in self.bias]
+        ws, bs = self.w_suffix, self.b_suffix
+        specs = [ParamSpec(f"{at[role]}{ws}", (rows, self.hidden_size)) for role, rows in self.stored.items()]
+        specs.append(ParamSpec(f"{at['o']}{ws}", (self.hidden_size, self.q_size)))
+        specs += [ParamSpec(f"{at[role]}{bs}", (rows,)) for role, rows in self.stored.items() if role in self.bias]
         if "o" in self.bias:
-            specs.append(ParamSpec(f"{at['o']}.bias", (self.hidden_size,)))
-        if self.qk_norm is not None:
+            specs.append(ParamSpec(f"{at['o']}{bs}", (self.hidden_size,)))
+        if self.qk_norm is not None and self.norm_weight:
             specs += [
                 ParamSpec(f"{at['q_norm']}.weight", (self.head_dim,), init=("normal", 0.1)),
                 ParamSpec(f"{at['k_norm']}.weight", (self.head_dim,), init=("normal", 0.1)),
@@ -73,17 +114,18 @@ class PagedAttention(Mixer):
         at = {role: f"{prefix}.{name}" for role, name in self.names.items()}
         # q, k and v rows are joined into one matrix, as the reference's loader
         # joins them (v3/crates/rvllm-loader/src/gemma4_load.rs:522,621-625).
-        parts = [tensors[f"{at[role]}.weight"].to(device=device, dtype=dtype) for role in self.stored]
+        ws, bs = self.w_suffix, self.b_suffix
+        parts = [tensors[f"{at[role]}{ws}"].to(device=device, dtype=dtype) for role in self.stored]
         self.w_qkv = decode_weight(torch.cat(parts, dim=0).contiguous(), self.tiled_weights)
-        self.w_o = decode_weight(tensors[f"{at['o']}.weight"].to(device=device, dtype=dtype).contiguous(),
+        self.w_o = decode_weight(tensors[f"{at['o']}{ws}"].to(device=device, dtype=dtype).contiguous(),
                                  self.tiled_weights)
         if self.bias & set(self.stored):  # projections without a bias of their own add zeros
             self.b_qkv = torch.cat([
-                tensors[f"{at[role]}.bias"].to(device=device, dtype=torch.float32) if role in self.bias
+                tensors[f"{at[role]}{bs}"].to(device=device, dtype=torch.float32) if role in self.bias
                 else torch.zeros(rows, dtype=torch.float32, device=device) for role, rows in self.stored.items()])
         if "o" in self.bias:
-            self.b_o = tensors[f"{at['o']}.bias"].to(device=device, dtype=torch.float32).contiguous()
-        if self.qk_norm is not None:
+            self.b_o = tensors[f"{at['o']}{bs}"].to(device=device, dtype=torch.float32).contiguous()
+        if self.qk_norm is not None and self.norm_weight:
             self.q_norm_w = tensors[f"{at['q_norm']}.weight"].to(device).contiguous()
             self.k_norm_w = tensors[f"{at['k_norm']}.weight"].to(device).contiguous()
             if self.q_norm_w.dtype != self.k_norm_w.dtype:
@@ -95,6 +137,8 @@ class PagedAttention(Mixer):
 
     # ---- run ---------------------------------------------------------
     def forward(self, x: torch.Tensor, step, cache: KVCacheView) -> torch.Tensor:
+        if self.general_path:
+            return self._forward_general(x, step, cache)
         n = x.shape[0]
         qkv = linear(x, self.w_qkv, sliced_ok=True)
         if self.b_qkv is not None:
@@ -114,6 +158,33 @@ class PagedAttention(Mixer):
         attn = torch.empty_like(q)
         ops.paged_attention(q, cache.k_pages, cache.v_pages, table, step, attn, self.num_heads, self.scale,
                             self.window)
+        out = linear(attn, self.w_o, sliced_ok=True)
+        return out if self.b_o is None else ops.add_bias(out, self.b_o)
+
+
+    def _forward_general(self, x: torch.Tensor, step, cache: KVCacheView) -> torch.Tensor:
+        """The variants: the rows of the fused projection hold q | k | (v) | (g)."""
+        n = x.shape[0]
+        proj = linear(x, self.w_qkv)
+        if self.b_qkv is not None:
+            proj = ops.add_bias(proj, self.b_qkv)
+        q = torch.empty((n, self.q_size), dtype=x.dtype, device=x.device)
+        table = step.block_tables[cache.group]
+        norm = self.qk_norm or {}
+        mode = ops.NORM_NONE if self.qk_norm is None else (
+            ops.NORM_AFTER_ROTATION if self.norm_after_rotation else ops.NORM_BEFORE_ROTATION)
+        k_col = self.q_size
+        v_col = None if self.values_from_keys else k_col + self.kv_size
+        ops.rotate_norm_write(
+            proj, 0, k_col, v_col, q, self.q_norm_w, self.k_norm_w, float(norm.get("eps", 0.0)),
+            1.0 if norm.get("unit_offset", False) else 0.0, mode, self.position.tables(step),
+            self.position.rotary_dim, step.positions, step.token_req, table, cache.k_pages, cache.v_pages,
+            self.num_heads, self.num_kv_heads, self.head_dim, write_kv=cache.writes)
+        attn = torch.empty_like(q)
+        ops.paged_attention(q, cache.k_pages, cache.v_pages, table, step, attn, self.num_heads, self.scale,
+                            self.window)
+        if self.gate:
+            ops.gate_mul_(attn, proj, proj.shape[1] - self.q_size, self.gate)
         out = linear(attn, self.w_o, sliced_ok=True)
         return out if self.b_o is None else ops.add_bias(out, self.b_o)
 

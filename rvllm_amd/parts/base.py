@@ -86,7 +86,27 @@ class StateNeed:
     dtype: torch.dtype = torch.float32
 
 
-CacheNeed = "KVNeed | StateNeed | None"
+CacheNeed = "KVNeed | StateNeed | tuple | None"
+
+
+def atomic_needs(need) -> tuple:
+    """The single needs (``KVNeed`` / ``StateNeed``) inside what a mixer declares: one of them, None, or a tuple of
+    these for a mixer that holds several mixers side by side (a tuple keeps a None for a member without a need,
+    so that its entries match the members)."""
+    if need is None:
+        return ()
+    if isinstance(need, (tuple, list)):
+        return tuple(a for member in need for a in atomic_needs(member))
+    return (need,)
+
+
+def reader_view(view):
+    """The read-only form of a layer's cache view, member by member for a tuple of views."""
+    if view is None:
+        return None
+    if isinstance(view, tuple):
+        return tuple(reader_view(v) for v in view)
+    return view.reader()
 
 
 @dataclasses.dataclass
@@ -191,6 +211,8 @@ class Mixer(Part):
     was left unreduced for the norm that follows (``ops.as_tensor`` reduces)."""
 
     def cache_need(self):
+        """``KVNeed``, ``StateNeed``, None, or a tuple of these (one entry a member mixer); ``forward`` gets the
+        matching view, or the tuple of views."""
         return None
 
     def forward(self, x: torch.Tensor, step: "StepBatch", cache) -> torch.Tensor:

@@ -10,7 +10,14 @@ v3/crates/rvllm-runtime/src/gemma4_layer_exec.rs:1-28):
 
 A block may hand the next block its entry norm already applied (``then``),
 which lets the kernel that adds the feed-forward branch also write the next
-layer's normed input.
+layer's normed input.  Parameters of ``sandwich``: ``norm_names`` (the four
+norms' names under the layer's prefix, the Gemma names if absent) and
+``layer_scale`` = (name, name) or None: one learned number a channel that the
+normed mixer branch, and one that the normed feed-forward branch, is multiplied
+by before it is added (x = x + ls1 * norm(mixer(..))).  A layer whose
+feed-forward is ``none`` has the first sublayer only and asks for the first two
+norms only.  The residual stream may be 32-bit under bf16 activations
+(``ModelSpec.residual_float32``); the norms then read the one and write the other.
 
 ``parallel``: one norm, both branches read its output, and their sum is added
 with a multiplier; the residual stream is 32-bit whatever the activations' type:
@@ -45,30 +52,61 @@ class SandwichBlock(Block):
         self.hidden_size = hidden_size
         self.mixer = MIXERS.build(layer.mixer, hidden_size=hidden_size)
         self.feed_forward = FEED_FORWARDS.build(layer.feed_forward, hidden_size=hidden_size)
-        self.norm_in, self.norm_post_mixer, self.norm_pre_ff, self.norm_post_ff = (
-            NORMS.build(layer.norm, width=hidden_size, name=name) for name in self.NORM_NAMES)
+        self.has_feed_forward = layer.feed_forward.kind != "none"
+        names = tuple(spec.get("norm_names") or self.NORM_NAMES)
+        if len(names) != 4:
+            raise ValueError("a sandwich has four norms: before and after the mixer, before and after the feed-forward")
+        if not self.has_feed_forward:
+            names = names[:2]
+        self.norms = [NORMS.build(layer.norm, width=hidden_size, name=name) for name in names]
+        self.norm_in, self.norm_post_mixer = self.norms[:2]
+        self.norm_pre_ff, self.norm_post_ff = self.norms[2:] if self.has_feed_forward else (None, None)
+        scale_names = spec.get("layer_scale")
+        self.scale_names = None if scale_names is None else tuple(str(n) for n in scale_names)
+        if self.scale_names is not None and len(self.scale_names) != 2:
+            raise ValueError("layer_scale names two tensors: the mixer branch's and the feed-forward branch's")
+        self.scale_mixer: Optional[torch.Tensor] = None
+        self.scale_ff: Optional[torch.Tensor] = None
 
     def parts(self):
-        return (self.mixer, self.feed_forward, self.norm_in, self.norm_post_mixer, self.norm_pre_ff,
-                self.norm_post_ff)
+        return (self.mixer, self.feed_forward, *self.norms)
 
     def param_specs(self, prefix: str) -> list[ParamSpec]:
-        return [s for part in self.parts() for s in part.param_specs(prefix)]
+        specs = [s for part in self.parts() for s in part.param_specs(prefix)]
+        if self.scale_names is not None:
+            used = self.scale_names if self.has_feed_forward else self.scale_names[:1]
+            specs += [ParamSpec(tensor_path(prefix, name), (self.hidden_size,), init=("normal_about", 1.0, 0.1))
+                      for name in used]
+        return specs
 
     def bind(self, tensors, prefix, device, dtype) -> None:
         for part in self.parts():
             part.bind(tensors, prefix, device, dtype)
+        if self.scale_names is not None:  # applied in 32-bit with the norm
+            self.scale_mixer = tensors[tensor_path(prefix, self.scale_names[0])].to(
+                device=device, dtype=torch.float32).contiguous()
+            if self.has_feed_forward:
+                self.scale_ff = tensors[tensor_path(prefix, self.scale_names[1])].to(
+                    device=device, dtype=torch.float32).contiguous()
 
     def entry_norm(self) -> Optional[Norm]:
         return self.norm_in
+
+    @staticmethod
+    def _add(norm: Norm, branch, x, then, scale):
+        if scale is None:
+            return norm.add_into(branch, x, then=then)
+        return norm.add_into(branch, x, then=then, scale=scale)
 
     def forward(self, x: torch.Tensor, step, cache, entered: Optional[torch.Tensor] = None,
                 then: Optional[Norm] = None) -> Optional[torch.Tensor]:
         h = entered if entered is not None else self.norm_in.forward(x)
         a = self.mixer.forward(h, step, cache)
-        h = self.norm_post_mixer.add_into(a, x, then=self.norm_pre_ff)
+        if not self.has_feed_forward:
+            return self._add(self.norm_post_mixer, a, x, then, self.scale_mixer)
+        h = self._add(self.norm_post_mixer, a, x, self.norm_pre_ff, self.scale_mixer)
         f = self.feed_forward.forward(h, step)
-        return self.norm_post_ff.add_into(f, x, then=then)
+        return self._add(self.norm_post_ff, f, x, then, self.scale_ff)
 
 
 class ParallelBlock(Block):

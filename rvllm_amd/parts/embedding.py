@@ -25,21 +25,23 @@ from .spec import PartSpec
 
 
 class ScaledEmbedding(Embedding):
-    """Parameters: ``scale`` (1 if absent) and ``name``, the table's name under
-    the model's prefix (``embed_tokens`` if absent)."""
+    """Parameters: ``scale`` (1 if absent), ``name``, the table's name under
+    the model's prefix (``embed_tokens`` if absent), and ``suffix``, what follows
+    the name (``.weight`` if absent).  The output may be a 32-bit residual stream."""
 
     def __init__(self, spec: PartSpec, *, hidden_size: int, vocab_size: int):
         self.hidden_size = hidden_size
         self.vocab_size = vocab_size
         self.scale = float(spec.get("scale", 1.0))
         self.name = str(spec.get("name", "embed_tokens"))
+        self.suffix = str(spec.get("suffix", ".weight"))
         self.table: Optional[torch.Tensor] = None
 
     def param_specs(self, prefix: str) -> list[ParamSpec]:
-        return [ParamSpec(f"{prefix}.{self.name}.weight", (self.vocab_size, self.hidden_size))]
+        return [ParamSpec(tensor_path(prefix, self.name) + self.suffix, (self.vocab_size, self.hidden_size))]
 
     def bind(self, tensors, prefix, device, dtype) -> None:
-        self.table = tensors[f"{prefix}.{self.name}.weight"].to(device=device, dtype=dtype).contiguous()
+        self.table = tensors[tensor_path(prefix, self.name) + self.suffix].to(device=device, dtype=dtype).contiguous()
 
     def forward(self, step, out: torch.Tensor) -> torch.Tensor:
         return ops.embed_gather(self.table, step.token_ids, self.scale, out)
@@ -77,7 +79,8 @@ class PositionalEmbedding(Embedding):
 
 class LMHead(Head):
     """Parameters: ``tied`` (the head reads the embedding's table, which must
-    then have a ``table``), ``softcap`` (None: off) and ``weight_name``, the
+    then have a ``table``), ``softcap`` (None: off), ``scale`` (a number the
+    logits are multiplied by, before any soft-cap; 1 if absent) and ``weight_name``, the
     whole name of an untied head's matrix (``lm_head.weight`` if absent: the
     reference looks it up under no prefix, gemma4_load.rs:431-436)."""
 
@@ -87,6 +90,7 @@ class LMHead(Head):
         self.tied = bool(spec.get("tied", True))
         cap = spec.get("softcap")
         self.softcap = None if cap is None else float(cap)
+        self.scale = float(spec.get("scale", 1.0))
         self.weight_name = str(spec.get("weight_name", "lm_head.weight"))
         self.embedding = embedding
         self.weight: Optional[torch.Tensor] = None
@@ -107,6 +111,8 @@ class LMHead(Head):
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         logits = linear(x, self.weight, out_dtype=torch.float32)
+        if self.scale != 1.0:
+            ops.scale_(logits, self.scale)
         if self.softcap is not None:
             ops.softcap_(logits, self.softcap)
         return logits

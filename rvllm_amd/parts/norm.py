@@ -5,6 +5,10 @@ eps is added to the mean inside the root; sum, root and product are 32-bit
 ``unit_offset`` selects the zero-centred form of the Gemma checkpoints, where
 the stored weight is the gain minus one.
 
+``rmsnorm`` takes ``suffix`` (what the tensor's name is followed by, ``.weight`` if
+absent).  Where the model keeps its residual stream in 32 bits and its
+activations in bf16, the norm reads the one and writes the other.
+
 ``rmsnorm_scalar``: the same with one number as the gain of the whole row,
 y = x * rsqrt(mean(x^2) + eps) * g.  Its input may be a residual stream that a
 bf16 model keeps in 32 bits; the output has the activations' type.  ``suffix``
@@ -29,22 +33,42 @@ class RMSNorm(Norm):
         self.name = name
         self.eps = float(spec["eps"])
         self.offset = 1.0 if spec.get("unit_offset", False) else 0.0
+        self.suffix = str(spec.get("suffix", ".weight"))
         self.weight: Optional[torch.Tensor] = None
+        self.out_dtype: Optional[torch.dtype] = None
+
+    def _tensor_name(self, prefix: str) -> str:
+        return tensor_path(prefix, self.name) + self.suffix
 
     def param_specs(self, prefix: str) -> list[ParamSpec]:
-        return [ParamSpec(f"{prefix}.{self.name}.weight", (self.width,), init=("normal", 0.1))]
+        return [ParamSpec(self._tensor_name(prefix), (self.width,), init=("normal", 0.1))]
 
     def bind(self, tensors, prefix, device, dtype) -> None:
         # The weight keeps the type it was loaded in (bf16, or 32-bit).
-        self.weight = tensors[f"{prefix}.{self.name}.weight"].to(device).contiguous()
+        self.weight = tensors[self._tensor_name(prefix)].to(device).contiguous()
+        self.out_dtype = dtype
 
     def forward(self, x: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+        if x.dtype != self.out_dtype:  # a 32-bit residual stream under bf16 activations
+            return ops.rmsnorm_cast(x, self.weight, self.eps, self.offset, self.out_dtype, out=out)
         return ops.rmsnorm(x, self.weight, self.eps, self.offset, out=out)
 
     def forward_rows(self, x: torch.Tensor, rows: torch.Tensor) -> torch.Tensor:
+        if x.dtype != self.out_dtype:
+            return ops.rmsnorm_cast(x, self.weight, self.eps, self.offset, self.out_dtype, rows=rows)
         return ops.rmsnorm(x, self.weight, self.eps, self.offset, rows=rows)
 
-    def add_into(self, branch, residual, then=None, then_out=None):
+    def add_into(self, branch, residual, then=None, then_out=None, scale=None):
+        """``scale``: one learned number a channel that the normed branch is multiplied by before it is added."""
+        if scale is not None or residual.dtype != self.out_dtype:
+            # the general kernel: a 32-bit stream whatever the branch's type, an optional scale
+            if residual.dtype != torch.float32:
+                raise ValueError("a scaled branch is added to a 32-bit residual stream")
+            if isinstance(then, RMSNorm):
+                return ops.add_rmsnorm_scaled(branch, self.weight, self.eps, self.offset, scale, residual, then.weight,
+                                              then.eps, then.offset)
+            ops.add_rmsnorm_scaled(branch, self.weight, self.eps, self.offset, scale, residual)
+            return then.forward(residual, out=then_out) if then is not None else None
         if then is None:
             return ops.add_rmsnorm(branch, self.weight, self.eps, self.offset, residual)
         if isinstance(then, RMSNorm):

@@ -8,6 +8,12 @@ global layers: the angle of position p becomes that of p / factor.  The table
 is computed in 64-bit and rounded to 32-bit once; the angle
 ``float(pos) * inv_freq[i]`` and its sine and cosine are 32-bit in the kernel
 that tabulates them for a step's tokens.
+
+``exponent_over`` is what the exponent divides by, ``head_dim`` (the default)
+or ``rotary_dim``: inv_freq[i] = theta^(-2i/rotary_dim).  ``pairing`` says which
+dimension turns with dimension i < rotary_dim/2: ``head_half`` (i + head_dim/2,
+the default) or ``rotary_half`` (i + rotary_dim/2, the rotated dimensions being
+the head's first ``rotary_dim``); the two agree where the whole head is rotated.
 """
 
 from __future__ import annotations
@@ -29,11 +35,16 @@ class RotaryEncoding(PositionEncoding):
         self.rotary_dim = int(spec.get("rotary_dim", head_dim))
         if self.rotary_dim % 2 or not 0 <= self.rotary_dim <= self.head_dim:
             raise ValueError(f"rotary_dim {self.rotary_dim} must be even and at most head_dim {self.head_dim}")
+        self.exponent_over = str(spec.get("exponent_over", "head_dim"))
+        self.pairing = str(spec.get("pairing", "head_half"))
+        if self.exponent_over not in ("head_dim", "rotary_dim") or self.pairing not in ("head_half", "rotary_half"):
+            raise ValueError(f"rope: exponent_over {self.exponent_over!r} / pairing {self.pairing!r} unknown")
         self._table: Optional[torch.Tensor] = None
 
     def inv_freq_host(self) -> torch.Tensor:
         i = torch.arange(self.rotary_dim // 2, dtype=torch.float64)
-        inv = self.theta ** (-2.0 * i / self.head_dim) / self.factor
+        over = self.head_dim if self.exponent_over == "head_dim" else self.rotary_dim
+        inv = self.theta ** (-2.0 * i / over) / self.factor
         return inv.to(torch.float32)
 
     def inv_freq(self, device) -> Optional[torch.Tensor]:
@@ -50,7 +61,7 @@ class RotaryEncoding(PositionEncoding):
         if self.rotary_dim == 0:
             return None
         shared = getattr(step, "shared", None)
-        key = ("rope", self.theta, self.factor, self.rotary_dim, self.head_dim)
+        key = ("rope", self.theta, self.factor, self.rotary_dim, self.head_dim, self.exponent_over)
         if shared is not None and key in shared:
             return shared[key]
         from ..kernels import ops
@@ -63,6 +74,8 @@ class RotaryEncoding(PositionEncoding):
 
 class NoPositionEncoding(PositionEncoding):
     """Queries and keys are left as they are."""
+
+    pairing = "head_half"
 
     def __init__(self, spec: PartSpec, *, head_dim: int):
         self.rotary_dim = 0
