@@ -75,6 +75,7 @@ def build_spec(cfg: RufedraConfig) -> ModelSpec:
             ff = PartSpec("gated_mlp", {
                 "intermediate_size": layer.mlp.ff, "activation": "gelu_tanh",
                 "names": {"gate": "mlp.gate", "up": "mlp.up", "down": "mlp.down"}, "weight_suffix": "",
+                "unrounded_output": True,
             })
         block = PartSpec("sandwich", {"norm_names": ("norm1", "norm1b", "norm2", "norm2b"),
                                       "layer_scale": ("ls1", "ls2")})

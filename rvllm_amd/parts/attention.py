@@ -34,7 +34,7 @@ import torch
 
 from ..kernels import ops
 from .base import KVCacheView, KVNeed, Mixer, ParamSpec
-from .linear import bias_roles, decode_weight, linear, tensor_names
+from .linear import bias_roles, decode_weight, linear, linear_unrounded, tensor_names
 from .registry import MIXERS, POSITION_ENCODINGS
 from .spec import PartSpec
 
@@ -185,8 +185,9 @@ class PagedAttention(Mixer):
                             self.window)
         if self.gate:
             ops.gate_mul_(attn, proj, proj.shape[1] - self.q_size, self.gate)
-        out = linear(attn, self.w_o, sliced_ok=True)
-        return out if self.b_o is None else ops.add_bias(out, self.b_o)
+        if self.b_o is None:
+            return linear_unrounded(attn, self.w_o)
+        return ops.add_bias(linear(attn, self.w_o, sliced_ok=True), self.b_o)
 
 
 MIXERS.register("attention", PagedAttention)

@@ -25,7 +25,7 @@ import torch
 
 from ..kernels import ops
 from .base import Mixer, ParamSpec, StateNeed, StateView
-from .linear import decode_weight, linear, tensor_names
+from .linear import decode_weight, linear, linear_unrounded, tensor_names
 from .registry import MIXERS
 from .spec import PartSpec
 
@@ -116,7 +116,7 @@ class GatedDeltaRule(Mixer):
         o = ops.delta_rule(qkv, 0, self.qk_size, qk, proj, self.a_col, self.b_col, self.A_log, self.dt_bias, slots,
                            self.s_off, step, self.heads, self.kv_heads, self.dim, self.vdim)
         y = ops.head_norm_gate(o, proj, self.g_col, self.norm_w, self.eps, self.heads, self.vdim, x.dtype)
-        return linear(y, self.w_o, sliced_ok=True)
+        return linear_unrounded(y, self.w_o)
 
 
 MIXERS.register("gated_delta_rule", GatedDeltaRule)

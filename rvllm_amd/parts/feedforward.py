@@ -11,7 +11,9 @@ layer's prefix, without ``.weight`` (the Gemma names if absent); a role
 ``gate_up`` names one stored matrix that holds the gate rows and then the up
 rows.  ``bias`` lists the projections that have a ``.bias`` (True: all).
 ``weight_suffix`` and ``bias_suffix`` are what a projection's name is followed
-by (``.weight`` and ``.bias`` if absent).
+by (``.weight`` and ``.bias`` if absent).  ``unrounded_output``: the down
+projection's 32-bit sums go on as they are (``linear.linear_unrounded``), for a
+block that adds its branches to a 32-bit residual stream.
 
 ``none`` is the feed-forward of a layer that has none: it adds nothing.
 """
@@ -22,7 +24,7 @@ import torch
 
 from ..kernels import ops
 from .base import FeedForward, ParamSpec
-from .linear import bias_roles, decode_weight, linear, tensor_names
+from .linear import bias_roles, decode_weight, linear, linear_unrounded, tensor_names
 from .registry import FEED_FORWARDS
 from .spec import PartSpec
 
@@ -42,6 +44,7 @@ class GatedMLP(FeedForward):
         inter = self.intermediate_size
         self.stored = {"gate_up": 2 * inter} if "gate_up" in self.names else {"gate": inter, "up": inter}
         self.bias = bias_roles(spec.get("bias"), [*self.stored, "down"])
+        self.unrounded_output = bool(spec.get("unrounded_output", False))
         self.w_gate_up = self.w_down = self.b_gate_up = self.b_down = None
         self.fours = False
 
@@ -94,6 +97,8 @@ class GatedMLP(FeedForward):
             if self.b_gate_up is not None:
                 gate_up = ops.add_bias(gate_up, self.b_gate_up)
             act = ops.gated_act(gate_up, self.activation, fours=self.fours)
+        if self.unrounded_output and self.b_down is None:
+            return linear_unrounded(act, self.w_down)
         out = linear(act, self.w_down, sliced_ok=True)
         return out if self.b_down is None else ops.add_bias(out, self.b_down)
 

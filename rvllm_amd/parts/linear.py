@@ -95,3 +95,18 @@ def linear(x: torch.Tensor, w, out: Optional[torch.Tensor] = None,
             return out
         return ops.gemm_plain(x, w, out)
     raise ops.KernelError(f"linear: unsupported dtypes x={x.dtype} w={w.dtype}")
+
+
+def linear_unrounded(x: torch.Tensor, w):
+    """A branch's last product for a consumer that takes ``ops.SlicedSums`` (the norm that adds a branch to a 32-bit
+    residual stream, the weighted sum of mixers side by side): the 32-bit sums are handed on as they are instead of
+    being rounded to bf16 in between.  Few rows: the unreduced K slices where the product has several; otherwise, and
+    for many rows, a 32-bit result as one slice.  A 32-bit engine's result is a plain tensor."""
+    if x.dtype is not torch.bfloat16:
+        return linear(x, w)
+    if x.shape[0] <= ops.SKINNY_MAX_ROWS:
+        fast = ops.gemm_bf16(x, w, None, out_dtype=torch.bfloat16, sliced_ok=True) if x.shape[0] > 0 else None
+        if isinstance(fast, ops.SlicedSums):
+            return fast
+    out = linear(x, w, out_dtype=torch.float32)
+    return ops.SlicedSums(out.view(1, *out.shape), torch.bfloat16)

@@ -21,7 +21,7 @@ import torch
 
 from ..kernels import ops
 from .base import Mixer, ParamSpec, StateNeed, StateView
-from .linear import decode_weight, linear, tensor_names
+from .linear import decode_weight, linear, linear_unrounded, tensor_names
 from .registry import MIXERS
 from .spec import PartSpec
 
@@ -89,7 +89,7 @@ class SelectiveScan(Mixer):
         dbc = linear(xc, self.w_x)  # [n, dt | B | C]
         dt = linear(dbc[:, :R], self.w_dt)
         y = ops.selective_scan(xc, proj, I, dt, self.dt_b, dbc, R, R + N, self.A_log, self.D, slots, self.s_off, step)
-        return linear(y, self.w_o, sliced_ok=True)
+        return linear_unrounded(y, self.w_o)
 
 
 MIXERS.register("selective_scan", SelectiveScan)
