@@ -3,7 +3,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--context 8192] [--layers L]
     python bench.py --workload 12b|27b [--requests N] [--layers L]     (another measurement, see WORKLOADS)
-    python bench.py --design pinorax [--size s|l] [--layers L]          (another measurement, see DESIGN_SIZES)
+    python bench.py --design pinorax|rufedra [--size s|l] [--layers L]  (another measurement, see DESIGN_SIZES)
 
 Default run: the layer sizes of the 4B-sized configuration (34 layers, 5
 sliding : 1 global, hidden 2560, 8 query / 4 key-value heads of 256, GeGLU
@@ -333,6 +333,44 @@ DESIGN_SIZES = {
 }
 
 
+# The Rufedra layers: in turn a gated delta rule layer without a feed-forward (``heads`` value heads of ``dim`` over
+# ``kv_heads`` query/key heads, short convolutions of ``conv`` taps) and a layer with two mixers side by side,
+# attention over a sliding window (``heads`` over ``kv_heads`` heads of ``dim``, half of a head rotated) beside a
+# selective scan (``inner`` channels of ``state`` states), with a dense feed-forward.  Beside it the dense decoder at
+# equal size: the same width, layers, vocabulary, heads and window in every layer, the same feed-forward in every
+# layer (the dense decoder has one in each, Rufedra in every second).
+RUFEDRA_SIZES = {
+    "s": dict(width=2048, heads=16, kv_heads=4, dim=128, window=1024, conv=4, inner=4096, state=16, dt_rank=128,
+              ff=8192, vocab=32000),
+    "l": dict(width=4096, heads=32, kv_heads=8, dim=128, window=1024, conv=4, inner=8192, state=16, dt_rank=256,
+              ff=12288, vocab=32000),
+}
+
+
+def rufedra_configs(size: dict, layers: int, positions: int):
+    from rvllm_amd.config.gemma3 import Gemma3Config
+    from rvllm_amd.config.rufedra import RufedraConfig
+
+    delta = {"type": "delta", "mlp": None, "mixer": {"heads": size["heads"], "kv_heads": size["kv_heads"],
+                                                      "dim": size["dim"], "vdim": size["dim"], "conv": size["conv"]}}
+    left = {"heads": size["heads"], "kv_heads": size["kv_heads"], "dim": size["dim"], "vdim": size["dim"],
+            "scale": size["dim"] ** -0.5, "mask": {"size": size["window"]},
+            "rot": {"dims": size["dim"] // 2, "base": 10000.0}}
+    right = {"inner": size["inner"], "state": size["state"], "dt_rank": size["dt_rank"], "conv": size["conv"]}
+    parallel = {"type": "parallel", "mlp": {"kind": "dense", "ff": size["ff"]},
+                "mixer": {"left": left, "right": right, "left_scale": 1.0, "right_scale": 1.0}}
+    rufedra = RufedraConfig.from_dict({
+        "architecture": "Rufedra", "vocab": size["vocab"], "width": size["width"], "embedding": {"scale": 1.0},
+        "norm": {"eps": 1e-6}, "logit_scale": 1.0, "layers": [delta if i % 2 == 0 else parallel for i in range(layers)],
+    }, "bench configuration")
+    dense = Gemma3Config.from_dict(dict(
+        GEMMA3_4B, num_hidden_layers=layers, hidden_size=size["width"], num_attention_heads=size["heads"],
+        num_key_value_heads=size["kv_heads"], head_dim=size["dim"], intermediate_size=size["ff"],
+        vocab_size=size["vocab"], query_pre_attn_scalar=size["dim"], max_position_embeddings=positions,
+        sliding_window=size["window"], layer_types=["sliding_attention"] * layers), "bench configuration")
+    return rufedra, dense
+
+
 def design_configs(size: dict, layers: int, positions: int):
     from rvllm_amd.config.gemma3 import Gemma3Config
     from rvllm_amd.config.pinorax import PinoraxConfig
@@ -357,7 +395,7 @@ def design_configs(size: dict, layers: int, positions: int):
 
 
 def run_design(args) -> int:
-    """Prefill and decode of the Pinorax design beside the dense decoder at equal size; one JSON line."""
+    """Prefill and decode of another design beside the dense decoder at equal size; one JSON line."""
     import torch
 
     from rvllm_amd.config.engine_config import EngineConfig
@@ -366,17 +404,19 @@ def run_design(args) -> int:
     from rvllm_amd.sampling.sampler import Sampler, SplitMix64
     import rvllm_amd.models  # noqa: F401
 
-    size = DESIGN_SIZES[args.size]
+    design = args.design
+    size = (RUFEDRA_SIZES if design == "rufedra" else DESIGN_SIZES)[args.size]
+    make_configs = rufedra_configs if design == "rufedra" else design_configs
     layers = args.layers if args.layers != FULL_LAYERS else 8
     context, T = args.context, args.prefill_tokens
     batches = [b for b in (8, 64) if not (args.no_points and b != 8)]
     steps_total = args.steps + args.warmup + 8
     positions = max(context + steps_total + 16, T)
-    out = {"metric": f"prefill and decode of Pinorax beside the dense decoder, size {args.size}", "unit": "ms",
+    out = {"metric": f"prefill and decode of {design.capitalize()} beside the dense decoder, size {args.size}", "unit": "ms",
            "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic: random weights, caches filled "
            "with random values, uniform token ids", "config": dict(size, layers=layers, context=context, prefill_tokens=T),
            "designs": {}}
-    for name, cfg in zip(("pinorax", "dense"), design_configs(size, layers, positions)):
+    for name, cfg in zip((design, "dense"), make_configs(size, layers, positions)):
         engine_cfg = EngineConfig(dtype=args.dtype, page_size=args.page_size, max_model_len=positions,
                                   max_num_seqs=max(batches), max_num_batched_tokens=max(T, max(batches)),
                                   max_prefill_chunk=T, max_cache_tokens=max(batches) * (context + steps_total + 16),
@@ -401,8 +441,8 @@ def run_design(args) -> int:
         import gc
         gc.collect()
         torch.cuda.empty_cache()
-    p, d = out["designs"]["pinorax"], out["designs"]["dense"]
-    out["pinorax_over_dense"] = {k: round(p[k] / d[k], 3) for k in p if k.endswith("_ms") and k in d}
+    p, d = out["designs"][design], out["designs"]["dense"]
+    out[f"{design}_over_dense"] = {k: round(p[k] / d[k], 3) for k in p if k.endswith("_ms") and k in d}
     print(json.dumps(out), flush=True)
     return 0
 
@@ -431,9 +471,10 @@ def main() -> int:
     ap.add_argument("--workload", choices=sorted(WORKLOADS), help="instead of the default run: an engine workload of a "
                     "larger configuration (requests through the scheduler); --requests and --layers shrink it")
     ap.add_argument("--requests", type=int, default=0)
-    ap.add_argument("--design", choices=["pinorax"], help="instead of the default run: prefill and decode of another "
+    ap.add_argument("--design", choices=["pinorax", "rufedra"], help="instead of the default run: prefill and decode of another "
                     "design of the framework beside the dense decoder at equal size (--size, --layers, --context)")
-    ap.add_argument("--size", choices=sorted(DESIGN_SIZES), default="s")
+    ap.add_argument("--size", choices=sorted(DESIGN_SIZES), default="s", help="of --design: s or l (see DESIGN_SIZES, "
+                    "RUFEDRA_SIZES)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this single-GPU engine", flush=True)

@@ -23,10 +23,34 @@ __device__ __forceinline__ float rec_softplus(float x) { return fmaxf(x, 0.f) + 
 __device__ __forceinline__ float rec_sigmoid(float x) { return 1.0f / (1.0f + expf(-x)); }
 __device__ __forceinline__ float rec_silu(float x) { return x / (1.0f + expf(-x)); }
 
-// Sum over the `lanes` (a power of two) neighbouring lanes that share a column or channel.
-__device__ __forceinline__ float rec_group_sum(float v, int lanes) {
-  for (int off = lanes >> 1; off > 0; off >>= 1) v += __shfl_xor(v, off, RV_WAVE);
+// Sum over the LANES (a power of two) neighbouring lanes that share a column or channel; every one of them gets it.
+// A token's work is one chain of dependent steps, and a wave often has its SIMD to itself, so the exchanges'
+// latency counts: within 16 lanes they are DPP moves between registers (pairs, then pairs of pairs, then the two
+// halves of 8 and of 16 mirrored, each half already holding its own sum in every lane), not trips through LDS.
+template <int CTRL>
+__device__ __forceinline__ float rec_dpp(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
+}
+template <int LANES>
+__device__ __forceinline__ float rec_group_sum(float v) {
+  if constexpr (LANES >= 2) v += rec_dpp<0xB1>(v);    // quad_perm [1,0,3,2]
+  if constexpr (LANES >= 4) v += rec_dpp<0x4E>(v);    // quad_perm [2,3,0,1]
+  if constexpr (LANES >= 8) v += rec_dpp<0x141>(v);   // row_half_mirror
+  if constexpr (LANES >= 16) v += rec_dpp<0x140>(v);  // row_mirror
+  if constexpr (LANES >= 32) v += __shfl_xor(v, 16, RV_WAVE);
+  if constexpr (LANES >= 64) v += __shfl_xor(v, 32, RV_WAVE);
   return v;
+}
+
+// The exponential of the scan's decay, once a state and token: the accurate one in a 32-bit engine; under bf16
+// activations the hardware's (base two, an error of about 1e-6), as the other kernels' activations there.
+template <typename T>
+__device__ __forceinline__ float rec_decay_exp(float x);
+template <>
+__device__ __forceinline__ float rec_decay_exp<float>(float x) { return expf(x); }
+template <>
+__device__ __forceinline__ float rec_decay_exp<bf16_t>(float x) {
+  return __builtin_amdgcn_exp2f(1.4426950408889634f * x);
 }
 
 // ---------------------------------------------------------------------------
@@ -168,107 +192,170 @@ extern "C" int rv_conv_state_update(hipStream_t stream, const void* in, int dtyp
 }
 
 // ---------------------------------------------------------------------------
-// Gated delta rule.  A column j of a head's S (its dk numbers) never meets another column, so `lanes` neighbouring
-// lanes own one: lane `sub` of them holds rows sub, sub + lanes, ... (PER at most).  A wave holds 64 / lanes
-// columns of one head of one request and walks the request's tokens of this step in order; the next token's
-// operands are asked for before this token's are used.
+// Gated delta rule.  A column j of a head's S (its dk numbers) never meets another column, so LANES neighbouring
+// lanes own one: lane `sub` of them holds rows sub * PER .. + PER.  A wave holds 64 / LANES columns of one head of
+// one request and walks the request's tokens of this step in order.  Going to memory for every token would cost a
+// round trip a token (the walk is a chain), so the tokens' operands come CHUNK at a time: all lanes read the chunk's
+// keys, queries, values and gate inputs side by side into registers while the chunk before is worked on, and put
+// them into LDS once that is done; decay and beta are worked out there, once a token.
 //   qkv  float [tokens, ld]: q of key head g at q_off + g dk, k at k_off + g dk, v of head h at v_off + h dv
 //   ab   T [tokens, ld_ab]: the decay's input a at a_col + h, beta's input at b_col + h
 //   g = exp(-exp(A_log[h]) softplus(a + dt_bias[h])),  beta = sigmoid(b)
-//   S    float [heads, dk, dv] at s_off of the request's slot
+//   S    float [heads, dv, dk] at s_off of the request's slot (a column's dk numbers side by side)
 //   out  float [tokens, heads dv]
+// What a token's sums are does not depend on CHUNK: the same multiply-adds in the same order.
 // ---------------------------------------------------------------------------
-template <typename T, int PER>
+template <typename T, int PER, int LANES, int CHUNK>
 __global__ void __launch_bounds__(RV_WAVE)
 delta_rule_kernel(const float* __restrict__ qkv, long long ld, int q_off, int k_off, int v_off,
                   const T* __restrict__ ab, long long ld_ab, int a_col, int b_col, const float* __restrict__ A_log,
                   const float* __restrict__ dt_bias, float* __restrict__ state, long long slot_stride,
                   long long s_off, const int* __restrict__ q_start, const int* __restrict__ state_slot,
-                  float* __restrict__ out, int heads, int kv_heads, int dk, int dv, int lanes) {
+                  float* __restrict__ out, int heads, int kv_heads, int dk, int dv) {
+  constexpr int COLS = RV_WAVE / LANES;
+  constexpr int DKP = PER * LANES;                          // the key size, padded
+  constexpr int NK = (CHUNK * DKP + RV_WAVE - 1) / RV_WAVE;  // keys (and queries) a lane brings in a chunk
+  constexpr int NV = (CHUNK * COLS + RV_WAVE - 1) / RV_WAVE;
+  __shared__ __attribute__((aligned(16))) float sk[CHUNK][DKP];
+  __shared__ __attribute__((aligned(16))) float sq[CHUNK][DKP];
+  __shared__ float sv[CHUNK][COLS];
+  __shared__ float sdecay[CHUNK], sbeta[CHUNK];
   const int lane = threadIdx.x;
-  const int cols = RV_WAVE / lanes;
-  const int sub = lane % lanes;
-  const int j = blockIdx.x * cols + lane / lanes;
+  const int sub = lane % LANES;
+  const int cl = lane / LANES;
+  const int j = blockIdx.x * COLS + cl;
   const int h = blockIdx.y;
   const int req = blockIdx.z;
   const int g = h / (heads / kv_heads);
   const bool col = j < dv;
   const int jj = col ? j : dv - 1;  // a lane past the last column works on a copy and writes nothing
-  float* S_mem = state + (long long)state_slot[req] * slot_stride + s_off + (long long)h * dk * dv + jj;
+  float* S_mem = state + (long long)state_slot[req] * slot_stride + s_off + ((long long)h * dv + jj) * dk + sub * PER;
+  const bool vec = (dk % 4 == 0) && (((uintptr_t)S_mem & 15) == 0);
   float S[PER];
 #pragma unroll
-  for (int e = 0; e < PER; ++e) {
-    const int i = e * lanes + sub;
-    S[e] = i < dk ? S_mem[(long long)i * dv] : 0.f;
+  for (int e = 0; e < PER; e += 4) {
+    if (vec && sub * PER + e < dk) {
+      const float4 v4 = *(const float4*)(S_mem + e);
+      S[e] = v4.x, S[e + 1] = v4.y, S[e + 2] = v4.z, S[e + 3] = v4.w;
+    } else {
+#pragma unroll
+      for (int u = 0; u < 4; ++u) S[e + u] = sub * PER + e + u < dk ? S_mem[e + u] : 0.f;
+    }
   }
   const float rate = -expf(A_log[h]);
   const float bias = dt_bias[h];
   const int t0 = q_start[req], t1 = q_start[req + 1];
-  float kk[PER], qq[PER], vv, a_in, b_in;
-  auto fetch = [&](int t, float (&k_)[PER], float (&q_)[PER], float& v_, float& a_, float& b_) {
-    const float* row = qkv + (long long)t * ld;
+  float rk[NK], rq[NK], rv[NV], ra = 0.f, rb = 0.f;
+  auto fetch = [&](int tb) {  // the chunk from token tb on, into registers
 #pragma unroll
-    for (int e = 0; e < PER; ++e) {
-      const int i = e * lanes + sub;
-      k_[e] = i < dk ? row[k_off + g * dk + i] : 0.f;
-      q_[e] = i < dk ? row[q_off + g * dk + i] : 0.f;
+    for (int r = 0; r < NK; ++r) {
+      const int idx = r * RV_WAVE + lane;
+      const int tok = idx / DKP, i = idx % DKP;
+      const bool ok = tok < CHUNK && tb + tok < t1 && i < dk;
+      const float* row = qkv + (long long)(ok ? tb + tok : t0) * ld + g * dk + (ok ? i : 0);
+      rk[r] = ok ? row[k_off] : 0.f;
+      rq[r] = ok ? row[q_off] : 0.f;
     }
-    v_ = row[v_off + h * dv + jj];
-    a_ = rv_to_float(ab[(long long)t * ld_ab + a_col + h]);
-    b_ = rv_to_float(ab[(long long)t * ld_ab + b_col + h]);
+#pragma unroll
+    for (int r = 0; r < NV; ++r) {
+      const int idx = r * RV_WAVE + lane;
+      const int tok = idx / COLS, c = idx % COLS;
+      const int jc = blockIdx.x * COLS + c;
+      const bool ok = tok < CHUNK && tb + tok < t1 && jc < dv;
+      rv[r] = ok ? qkv[(long long)(tb + tok) * ld + v_off + h * dv + jc] : 0.f;
+    }
+    if (lane < CHUNK && tb + lane < t1) {
+      ra = rv_to_float(ab[(long long)(tb + lane) * ld_ab + a_col + h]);
+      rb = rv_to_float(ab[(long long)(tb + lane) * ld_ab + b_col + h]);
+    }
   };
-  if (t0 < t1) fetch(t0, kk, qq, vv, a_in, b_in);
-  for (int t = t0; t < t1; ++t) {
-    float nk[PER], nq[PER], nv = 0.f, na = 0.f, nb = 0.f;
-    if (t + 1 < t1) fetch(t + 1, nk, nq, nv, na, nb);
-    const float decay = expf(rate * rec_softplus(a_in + bias));
-    const float beta = rec_sigmoid(b_in);
-    float dot = 0.f;
+  auto stage = [&]() {  // the registers into LDS
 #pragma unroll
-    for (int e = 0; e < PER; ++e) {
-      S[e] *= decay;
-      dot = fmaf(S[e], kk[e], dot);
+    for (int r = 0; r < NK; ++r) {
+      const int idx = r * RV_WAVE + lane;
+      if (idx < CHUNK * DKP) (&sk[0][0])[idx] = rk[r], (&sq[0][0])[idx] = rq[r];
     }
-    dot = rec_group_sum(dot, lanes);
-    const float u = beta * (vv - dot);
-    float o = 0.f;
 #pragma unroll
-    for (int e = 0; e < PER; ++e) {
-      S[e] = fmaf(kk[e], u, S[e]);
-      o = fmaf(S[e], qq[e], o);
+    for (int r = 0; r < NV; ++r) {
+      const int idx = r * RV_WAVE + lane;
+      if (idx < CHUNK * COLS) (&sv[0][0])[idx] = rv[r];
     }
-    o = rec_group_sum(o, lanes);
-    if (col && sub == 0) out[(long long)t * heads * dv + h * dv + j] = o;
-    if (t + 1 < t1) {
+    if (lane < CHUNK) {
+      sdecay[lane] = expf(rate * rec_softplus(ra + bias));
+      sbeta[lane] = rec_sigmoid(rb);
+    }
+  };
+  if (t0 < t1) fetch(t0);
+  for (int tb = t0; tb < t1; tb += CHUNK) {
+    __syncthreads();  // the chunk before has been read
+    stage();
+    __syncthreads();
+    if (tb + CHUNK < t1) fetch(tb + CHUNK);
+    const int n = min(CHUNK, t1 - tb);
+    for (int t = 0; t < n; ++t) {
+      float kk[PER], qq[PER];
 #pragma unroll
-      for (int e = 0; e < PER; ++e) kk[e] = nk[e], qq[e] = nq[e];
-      vv = nv, a_in = na, b_in = nb;
+      for (int e = 0; e < PER; e += 4) {
+        const float4 k4 = *(const float4*)&sk[t][sub * PER + e];
+        const float4 q4 = *(const float4*)&sq[t][sub * PER + e];
+        kk[e] = k4.x, kk[e + 1] = k4.y, kk[e + 2] = k4.z, kk[e + 3] = k4.w;
+        qq[e] = q4.x, qq[e + 1] = q4.y, qq[e + 2] = q4.z, qq[e + 3] = q4.w;
+      }
+      const float decay = sdecay[t];
+      const float beta = sbeta[t];
+      const float vv = sv[t][cl];
+      float dot = 0.f;
+#pragma unroll
+      for (int e = 0; e < PER; ++e) {
+        S[e] *= decay;
+        dot = fmaf(S[e], kk[e], dot);
+      }
+      dot = rec_group_sum<LANES>(dot);
+      const float u = beta * (vv - dot);
+      float o = 0.f;
+#pragma unroll
+      for (int e = 0; e < PER; ++e) {
+        S[e] = fmaf(kk[e], u, S[e]);
+        o = fmaf(S[e], qq[e], o);
+      }
+      o = rec_group_sum<LANES>(o);
+      if (col && sub == 0) out[(long long)(tb + t) * heads * dv + h * dv + j] = o;
     }
   }
   if (col) {
 #pragma unroll
-    for (int e = 0; e < PER; ++e) {
-      const int i = e * lanes + sub;
-      if (i < dk) S_mem[(long long)i * dv] = S[e];
+    for (int e = 0; e < PER; e += 4) {
+      if (vec && sub * PER + e < dk) {
+        *(float4*)(S_mem + e) = make_float4(S[e], S[e + 1], S[e + 2], S[e + 3]);
+      } else {
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+          if (sub * PER + e + u < dk) S_mem[e + u] = S[e + u];
+      }
     }
   }
 }
 
-#define REC_DELTA_PER_MAX 16
+#define REC_DELTA_PER 8       // rows of a column a lane holds, while up to 16 lanes share the column
+#define REC_DELTA_PER_MAX 16  // ... and beyond
 
 // How many lanes share a column of S for this key size: the fewest (a power of two) that leave a lane at most
-// REC_DELTA_PER_MAX rows.  A function of dk alone, so that a token's sums are added in one order always.
+// REC_DELTA_PER rows, up to 16 lanes (a prompt of one request then has a wave for every SIMD at the sizes in use,
+// and the sums stay within a DPP row); larger keys take up to REC_DELTA_PER_MAX rows a lane.  A function of dk
+// alone, so that a token's sums are added in one order always.
 extern "C" int rv_delta_rule_lanes(int dk) {
   int lanes = 1;
+  while (lanes < 16 && rv_div_up(dk, lanes) > REC_DELTA_PER) lanes *= 2;
   while (lanes < RV_WAVE && rv_div_up(dk, lanes) > REC_DELTA_PER_MAX) lanes *= 2;
   return lanes;
 }
 
+// `longest`: the most tokens a request brings in this step (the size of the chunks is chosen by it).
 extern "C" int rv_delta_rule(hipStream_t stream, const float* qkv, long long ld, int q_off, int k_off, int v_off,
                              const void* ab, int dtype, long long ld_ab, int a_col, int b_col, const float* A_log,
                              const float* dt_bias, float* state, long long slot_stride, long long s_off,
                              const int* q_start, const int* state_slot, float* out, int num_requests, int heads,
-                             int kv_heads, int dk, int dv) {
+                             int kv_heads, int dk, int dv, int longest) {
   RV_CHECK(qkv && ab && A_log && dt_bias && state && q_start && state_slot && out, "delta_rule: null argument");
   RV_CHECK(heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && dk > 0 && dv > 0 && num_requests >= 0,
            "delta_rule: bad sizes heads=%d kv_heads=%d dk=%d dv=%d", heads, kv_heads, dk, dv);
@@ -277,27 +364,43 @@ extern "C" int rv_delta_rule(hipStream_t stream, const float* qkv, long long ld,
   RV_CHECK(per <= REC_DELTA_PER_MAX, "delta_rule: a key size of %d is more than %d", dk, REC_DELTA_PER_MAX * RV_WAVE);
   if (num_requests == 0) return 0;
   dim3 grid(rv_div_up(dv, RV_WAVE / lanes), heads, num_requests), block(RV_WAVE);
-#define RV_DR(T, PER)                                                                                                \
-  delta_rule_kernel<T, PER><<<grid, block, 0, stream>>>(qkv, ld, q_off, k_off, v_off, (const T*)ab, ld_ab, a_col,    \
-                                                        b_col, A_log, dt_bias, state, slot_stride, s_off, q_start,   \
-                                                        state_slot, out, heads, kv_heads, dk, dv, lanes)
-#define RV_DR_T(T)                \
-  do {                            \
-    if (per <= 4) RV_DR(T, 4);    \
-    else if (per <= 8) RV_DR(T, 8); \
-    else RV_DR(T, 16);            \
+  const bool few = longest <= 2;  // decoded tokens: small chunks, little LDS, more waves a CU
+#define RV_DR(T, PER, LANES, CHUNK)                                                                             \
+  delta_rule_kernel<T, PER, LANES, CHUNK><<<grid, block, 0, stream>>>(                                          \
+      qkv, ld, q_off, k_off, v_off, (const T*)ab, ld_ab, a_col, b_col, A_log, dt_bias, state, slot_stride, s_off, \
+      q_start, state_slot, out, heads, kv_heads, dk, dv)
+  // chunks of up to 16 tokens while a chunk's keys stay within 2048 numbers (32 registers a lane)
+#define RV_DR_L(T, PER, LANES, CHUNK)          \
+  do {                                         \
+    if (few) RV_DR(T, PER, LANES, 2);          \
+    else RV_DR(T, PER, LANES, CHUNK);          \
+  } while (0)
+#define RV_DR_T(T)                                         \
+  do {                                                     \
+    if (lanes == 1 && per <= 4) RV_DR_L(T, 4, 1, 16);      \
+    else if (lanes == 1) RV_DR_L(T, 8, 1, 16);             \
+    else if (lanes == 2) RV_DR_L(T, 8, 2, 16);             \
+    else if (lanes == 4) RV_DR_L(T, 8, 4, 16);             \
+    else if (lanes == 8) RV_DR_L(T, 8, 8, 16);             \
+    else if (lanes == 16 && per <= 8) RV_DR_L(T, 8, 16, 16); \
+    else if (lanes == 16) RV_DR_L(T, 16, 16, 8);           \
+    else if (lanes == 32) RV_DR_L(T, 16, 32, 4);           \
+    else RV_DR_L(T, 16, 64, 2);                            \
   } while (0)
   if (dtype == RV_F32) RV_DR_T(float);
   else if (dtype == RV_BF16) RV_DR_T(bf16_t);
   else return rv_fail("delta_rule: unsupported dtype %d", dtype);
 #undef RV_DR_T
+#undef RV_DR_L
 #undef RV_DR
   RV_LAUNCH_CHECK("delta_rule");
   return 0;
 }
 
 // ---------------------------------------------------------------------------
-// Selective scan.  `lanes` neighbouring lanes own a channel: lane `sub` holds the states sub, sub + lanes, ...
+// Selective scan.  LANES neighbouring lanes own a channel: lane `sub` holds the states sub * PER .. + PER.  A wave
+// holds 64 / LANES channels of one request and walks its tokens of this step in order, CHUNK at a time through
+// registers and LDS as the delta rule above; the step sizes and the gates' silu are worked out once a token there.
 //   x    T [tokens, ld_x]    the convolved, activated input      z   T [tokens, ld_z]   the gate's input
 //   dt   T [tokens, ld_dt]   the step's projection; step = softplus(dt + dt_bias[c])
 //   bc   T [tokens, ld_bc]   B at b_col, C at c_col, `n_state` each
@@ -305,81 +408,114 @@ extern "C" int rv_delta_rule(hipStream_t stream, const float* qkv, long long ld,
 //   S    float [channels, n_state] at s_off of the request's slot
 //   out  T [tokens, channels] = (S . C + D x) silu(z)
 // ---------------------------------------------------------------------------
-template <typename T, int PER>
+template <typename T, int PER, int LANES, int CHUNK>
 __global__ void __launch_bounds__(RV_WAVE)
 selective_scan_kernel(const T* __restrict__ x, long long ld_x, const T* __restrict__ z, long long ld_z,
                       const T* __restrict__ dt, long long ld_dt, const float* __restrict__ dt_bias,
                       const T* __restrict__ bc, long long ld_bc, int b_col, int c_col,
                       const float* __restrict__ A_log, const float* __restrict__ D, float* __restrict__ state,
                       long long slot_stride, long long s_off, const int* __restrict__ q_start,
-                      const int* __restrict__ state_slot, T* __restrict__ out, int channels, int n_state, int lanes) {
+                      const int* __restrict__ state_slot, T* __restrict__ out, int channels, int n_state) {
+  constexpr int CPW = RV_WAVE / LANES;  // channels a wave
+  constexpr int NP = PER * LANES;       // the states, padded
+  constexpr int NB = (CHUNK * NP + RV_WAVE - 1) / RV_WAVE;
+  constexpr int NX = (CHUNK * CPW + RV_WAVE - 1) / RV_WAVE;
+  __shared__ __attribute__((aligned(16))) float sB[CHUNK][NP];
+  __shared__ __attribute__((aligned(16))) float sC[CHUNK][NP];
+  __shared__ float sx[CHUNK][CPW], sg[CHUNK][CPW], sstep[CHUNK][CPW];
   const int lane = threadIdx.x;
-  const int per_wave = RV_WAVE / lanes;
-  const int sub = lane % lanes;
-  const int ch = blockIdx.x * per_wave + lane / lanes;
+  const int sub = lane % LANES;
+  const int cl = lane / LANES;
+  const int ch0 = blockIdx.x * CPW;
+  const int ch = ch0 + cl;
   const int req = blockIdx.y;
   const bool live = ch < channels;
   const int c = live ? ch : channels - 1;
-  float* S_mem = state + (long long)state_slot[req] * slot_stride + s_off + (long long)c * n_state;
+  float* S_mem = state + (long long)state_slot[req] * slot_stride + s_off + (long long)c * n_state + sub * PER;
   float S[PER], A[PER];
 #pragma unroll
   for (int e = 0; e < PER; ++e) {
-    const int n = e * lanes + sub;
-    S[e] = n < n_state ? S_mem[n] : 0.f;
+    const int n = sub * PER + e;
+    S[e] = n < n_state ? S_mem[e] : 0.f;
     A[e] = n < n_state ? -expf(A_log[(long long)c * n_state + n]) : 0.f;
   }
-  const float bias = dt_bias[c];
   const float skip = D[c];
   const int t0 = q_start[req], t1 = q_start[req + 1];
-  float Bn[PER], Cn[PER], xv, zv, dv;
-  auto fetch = [&](int t, float (&B_)[PER], float (&C_)[PER], float& x_, float& z_, float& d_) {
-    const T* row = bc + (long long)t * ld_bc;
+  float rB[NB], rC[NB], rx[NX], rz[NX], rd[NX];
+  auto fetch = [&](int tb) {
 #pragma unroll
-    for (int e = 0; e < PER; ++e) {
-      const int n = e * lanes + sub;
-      B_[e] = n < n_state ? rv_to_float(row[b_col + n]) : 0.f;
-      C_[e] = n < n_state ? rv_to_float(row[c_col + n]) : 0.f;
+    for (int r = 0; r < NB; ++r) {
+      const int idx = r * RV_WAVE + lane;
+      const int tok = idx / NP, n = idx % NP;
+      const bool ok = tok < CHUNK && tb + tok < t1 && n < n_state;
+      const T* row = bc + (long long)(ok ? tb + tok : t0) * ld_bc + (ok ? n : 0);
+      rB[r] = ok ? rv_to_float(row[b_col]) : 0.f;
+      rC[r] = ok ? rv_to_float(row[c_col]) : 0.f;
     }
-    x_ = rv_to_float(x[(long long)t * ld_x + c]);
-    z_ = rv_to_float(z[(long long)t * ld_z + c]);
-    d_ = rv_to_float(dt[(long long)t * ld_dt + c]);
+#pragma unroll
+    for (int r = 0; r < NX; ++r) {
+      const int idx = r * RV_WAVE + lane;
+      const int tok = idx / CPW, cc = ch0 + idx % CPW;
+      const bool ok = tok < CHUNK && tb + tok < t1 && cc < channels;
+      const long long t = ok ? tb + tok : t0;
+      const int c_ = ok ? cc : 0;
+      rx[r] = ok ? rv_to_float(x[t * ld_x + c_]) : 0.f;
+      rz[r] = ok ? rv_to_float(z[t * ld_z + c_]) : 0.f;
+      rd[r] = ok ? rv_to_float(dt[t * ld_dt + c_]) + dt_bias[c_] : 0.f;
+    }
   };
-  if (t0 < t1) fetch(t0, Bn, Cn, xv, zv, dv);
-  for (int t = t0; t < t1; ++t) {
-    float nB[PER], nC[PER], nx = 0.f, nz = 0.f, nd = 0.f;
-    if (t + 1 < t1) fetch(t + 1, nB, nC, nx, nz, nd);
-    const float step = rec_softplus(dv + bias);
-    const float sx = step * xv;
-    float y = 0.f;
+  auto stage = [&]() {
 #pragma unroll
-    for (int e = 0; e < PER; ++e) {
-      S[e] = fmaf(expf(step * A[e]), S[e], sx * Bn[e]);
-      y = fmaf(S[e], Cn[e], y);
+    for (int r = 0; r < NB; ++r) {
+      const int idx = r * RV_WAVE + lane;
+      if (idx < CHUNK * NP) (&sB[0][0])[idx] = rB[r], (&sC[0][0])[idx] = rC[r];
     }
-    y = rec_group_sum(y, lanes);
-    y = fmaf(skip, xv, y);
-    if (live && sub == 0) out[(long long)t * channels + ch] = rv_from_float<T>(y * rec_silu(zv));
-    if (t + 1 < t1) {
 #pragma unroll
-      for (int e = 0; e < PER; ++e) Bn[e] = nB[e], Cn[e] = nC[e];
-      xv = nx, zv = nz, dv = nd;
+    for (int r = 0; r < NX; ++r) {
+      const int idx = r * RV_WAVE + lane;
+      if (idx < CHUNK * CPW) {
+        (&sx[0][0])[idx] = rx[r];
+        (&sg[0][0])[idx] = rec_silu(rz[r]);
+        (&sstep[0][0])[idx] = rec_softplus(rd[r]);
+      }
+    }
+  };
+  if (t0 < t1) fetch(t0);
+  for (int tb = t0; tb < t1; tb += CHUNK) {
+    __syncthreads();
+    stage();
+    __syncthreads();
+    if (tb + CHUNK < t1) fetch(tb + CHUNK);
+    const int n_tok = min(CHUNK, t1 - tb);
+    for (int t = 0; t < n_tok; ++t) {
+      const float step = sstep[t][cl];
+      const float xv = sx[t][cl];
+      const float sx_ = step * xv;
+      float y = 0.f;
+#pragma unroll
+      for (int e = 0; e < PER; ++e) {
+        S[e] = fmaf(rec_decay_exp<T>(step * A[e]), S[e], sx_ * sB[t][sub * PER + e]);
+        y = fmaf(S[e], sC[t][sub * PER + e], y);
+      }
+      y = rec_group_sum<LANES>(y);
+      y = fmaf(skip, xv, y);
+      if (live && sub == 0) out[(long long)(tb + t) * channels + ch] = rv_from_float<T>(y * sg[t][cl]);
     }
   }
   if (live) {
 #pragma unroll
-    for (int e = 0; e < PER; ++e) {
-      const int n = e * lanes + sub;
-      if (n < n_state) S_mem[n] = S[e];
-    }
+    for (int e = 0; e < PER; ++e)
+      if (sub * PER + e < n_state) S_mem[e] = S[e];
   }
 }
 
-#define REC_SCAN_PER 4
+#define REC_SCAN_PER_MAX 4
 
-// Lanes that share a channel: the fewest (a power of two) that leave a lane at most REC_SCAN_PER states.
+// Lanes that share a channel: one a state up to 64 (every state costs an exponential a token, and a prompt of one
+// request wants a wave for every SIMD), then up to REC_SCAN_PER_MAX states a lane.
 extern "C" int rv_selective_scan_lanes(int n_state) {
   int lanes = 1;
-  while (lanes < RV_WAVE && rv_div_up(n_state, lanes) > REC_SCAN_PER) lanes *= 2;
+  while (lanes < RV_WAVE && lanes < n_state) lanes *= 2;
   return lanes;
 }
 
@@ -388,22 +524,43 @@ extern "C" int rv_selective_scan(hipStream_t stream, const void* x, long long ld
                                  long long ld_bc, int b_col, int c_col, const float* A_log, const float* D,
                                  float* state, long long slot_stride, long long s_off, const int* q_start,
                                  const int* state_slot, void* out, int dtype, int num_requests, int channels,
-                                 int n_state) {
+                                 int n_state, int longest) {
   RV_CHECK(x && z && dt && dt_bias && bc && A_log && D && state && q_start && state_slot && out,
            "selective_scan: null argument");
   RV_CHECK(channels > 0 && n_state > 0 && num_requests >= 0, "selective_scan: bad sizes");
   const int lanes = rv_selective_scan_lanes(n_state);
-  RV_CHECK(rv_div_up(n_state, lanes) <= REC_SCAN_PER, "selective_scan: %d states a channel are more than %d", n_state,
-           REC_SCAN_PER * RV_WAVE);
+  const int per = rv_div_up(n_state, lanes);
+  RV_CHECK(per <= REC_SCAN_PER_MAX, "selective_scan: %d states a channel are more than %d", n_state,
+           REC_SCAN_PER_MAX * RV_WAVE);
   if (num_requests == 0) return 0;
   dim3 grid(rv_div_up(channels, RV_WAVE / lanes), num_requests), block(RV_WAVE);
-#define RV_SS(T)                                                                                                   \
-  selective_scan_kernel<T, REC_SCAN_PER><<<grid, block, 0, stream>>>(                                              \
+  const bool few = longest <= 2;
+#define RV_SS(T, PER, LANES, CHUNK)                                                                                \
+  selective_scan_kernel<T, PER, LANES, CHUNK><<<grid, block, 0, stream>>>(                                         \
       (const T*)x, ld_x, (const T*)z, ld_z, (const T*)dt, ld_dt, dt_bias, (const T*)bc, ld_bc, b_col, c_col, A_log, \
-      D, state, slot_stride, s_off, q_start, state_slot, (T*)out, channels, n_state, lanes)
-  if (dtype == RV_F32) RV_SS(float);
-  else if (dtype == RV_BF16) RV_SS(bf16_t);
+      D, state, slot_stride, s_off, q_start, state_slot, (T*)out, channels, n_state)
+#define RV_SS_L(T, PER, LANES, CHUNK)     \
+  do {                                    \
+    if (few) RV_SS(T, PER, LANES, 2);     \
+    else RV_SS(T, PER, LANES, CHUNK);     \
+  } while (0)
+#define RV_SS_T(T)                                    \
+  do {                                                \
+    if (lanes == 1) RV_SS_L(T, 1, 1, 16);             \
+    else if (lanes == 2) RV_SS_L(T, 1, 2, 16);        \
+    else if (lanes == 4) RV_SS_L(T, 1, 4, 16);        \
+    else if (lanes == 8) RV_SS_L(T, 1, 8, 16);        \
+    else if (lanes == 16) RV_SS_L(T, 1, 16, 16);      \
+    else if (lanes == 32) RV_SS_L(T, 1, 32, 16);      \
+    else if (per <= 1) RV_SS_L(T, 1, 64, 16);         \
+    else if (per <= 2) RV_SS_L(T, 2, 64, 8);          \
+    else RV_SS_L(T, 4, 64, 4);                        \
+  } while (0)
+  if (dtype == RV_F32) RV_SS_T(float);
+  else if (dtype == RV_BF16) RV_SS_T(bf16_t);
   else return rv_fail("selective_scan: unsupported dtype %d", dtype);
+#undef RV_SS_T
+#undef RV_SS_L
 #undef RV_SS
   RV_LAUNCH_CHECK("selective_scan");
   return 0;

@@ -49,12 +49,40 @@ extern "C" int rv_rmsnorm_cast(hipStream_t stream, const void* x, int x_dtype, c
 template <typename T>
 __device__ __forceinline__ float rs_branch(const void* p, int slices, long long stride, size_t at) {
   if (slices == 0) return rv_to_float(((const T*)p)[at]);
+  const float* q = (const float*)p + at;
   float v = 0.f;
-  for (int s = 0; s < slices; ++s) v += ((const float*)p)[(size_t)s * stride + at];
+  int s = 0;
+  for (; s + 4 <= slices; s += 4) {  // four reads on their way at a time, added in the slices' order
+    const float a = q[(size_t)s * stride], b = q[(size_t)(s + 1) * stride], c = q[(size_t)(s + 2) * stride],
+                d = q[(size_t)(s + 3) * stride];
+    v = (((v + a) + b) + c) + d;
+  }
+  for (; s < slices; ++s) v += q[(size_t)s * stride];
   return v;
 }
 
-template <typename T>
+// V values side by side (1, or 4 where rows and slices start on 16-byte boundaries) of a branch.
+template <typename T, int V>
+__device__ __forceinline__ void rs_load_branch(const void* p, bool sliced, size_t at, float* out) {
+  if (sliced || sizeof(T) == 4) {
+    if constexpr (V == 4) {
+      const float4 q = *(const float4*)((const float*)p + at);
+      out[0] = q.x, out[1] = q.y, out[2] = q.z, out[3] = q.w;
+    } else {
+      out[0] = ((const float*)p)[at];
+    }
+  } else if constexpr (V == 4) {
+    const uint2 q = *(const uint2*)((const uint16_t*)p + at);
+    out[0] = __uint_as_float(q.x << 16), out[1] = __uint_as_float(q.x & 0xffff0000u);
+    out[2] = __uint_as_float(q.y << 16), out[3] = __uint_as_float(q.y & 0xffff0000u);
+  } else {
+    out[0] = rv_to_float(((const T*)p)[at]);
+  }
+}
+
+// E: groups of V values a thread keeps in registers (its share of a row of up to E * V * RS_THREADS numbers); 0: any
+// width, the branch is read twice.  The reads of all a thread's groups are on their way together, slice after slice.
+template <typename T, int E, int V>
 __global__ void __launch_bounds__(RS_THREADS)
 add_rmsnorm_scaled_kernel(const void* __restrict__ branch, int slices, long long slice_stride,
                           const void* __restrict__ w_post, int w_post_f32, const void* __restrict__ scale,
@@ -63,27 +91,90 @@ add_rmsnorm_scaled_kernel(const void* __restrict__ branch, int slices, long long
                           float offset_next) {
   __shared__ float scratch[16];
   const size_t row0 = (size_t)blockIdx.x * width;
+  constexpr int N = E > 0 ? E : 1;
+  float val[N][V], res[N][V], gain[N][V];
   float ss = 0.f;
-  for (int i = threadIdx.x; i < width; i += RS_THREADS) {
-    const float v = rs_branch<T>(branch, slices, slice_stride, row0 + i);
-    ss = fmaf(v, v, ss);
+  if constexpr (E > 0) {
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+      const int i = (e * RS_THREADS + threadIdx.x) * V;
+#pragma unroll
+      for (int v = 0; v < V; ++v) val[e][v] = res[e][v] = gain[e][v] = 0.f;
+      if (i < width) {
+        rs_load_branch<float, V>(x, false, row0 + i, res[e]);
+#pragma unroll
+        for (int v = 0; v < V; ++v)
+          gain[e][v] = (offset + rv_load_w(w_post, w_post_f32, i + v)) * (scale ? rv_load_w(scale, scale_f32, i + v) : 1.0f);
+      }
+    }
+    const int rounds = slices > 0 ? slices : 1;
+    for (int s = 0; s < rounds; ++s) {
+      float part[E][V];
+#pragma unroll
+      for (int e = 0; e < E; ++e) {
+        const int i = (e * RS_THREADS + threadIdx.x) * V;
+#pragma unroll
+        for (int v = 0; v < V; ++v) part[e][v] = 0.f;
+        if (i < width) rs_load_branch<T, V>(branch, slices > 0, (size_t)s * slice_stride + row0 + i, part[e]);
+      }
+#pragma unroll
+      for (int e = 0; e < E; ++e)
+#pragma unroll
+        for (int v = 0; v < V; ++v) val[e][v] += part[e][v];
+    }
+#pragma unroll
+    for (int e = 0; e < E; ++e)
+#pragma unroll
+      for (int v = 0; v < V; ++v) ss = fmaf(val[e][v], val[e][v], ss);
+  } else {
+    for (int i = threadIdx.x; i < width; i += RS_THREADS) {
+      const float v = rs_branch<T>(branch, slices, slice_stride, row0 + i);
+      ss = fmaf(v, v, ss);
+    }
   }
   ss = rv_block_sum(ss, scratch);
   const float inv = 1.0f / sqrtf(ss / (float)width + eps);
   float ss2 = 0.f;
-  for (int i = threadIdx.x; i < width; i += RS_THREADS) {
-    float v = rs_branch<T>(branch, slices, slice_stride, row0 + i) * inv * (offset + rv_load_w(w_post, w_post_f32, i));
-    if (scale) v *= rv_load_w(scale, scale_f32, i);
-    const float r = x[row0 + i] + v;
-    x[row0 + i] = r;
-    ss2 = fmaf(r, r, ss2);
+  if constexpr (E > 0) {
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+      const int i = (e * RS_THREADS + threadIdx.x) * V;
+      if (i < width) {
+#pragma unroll
+        for (int v = 0; v < V; ++v) {
+          res[e][v] = res[e][v] + val[e][v] * inv * gain[e][v];
+          ss2 = fmaf(res[e][v], res[e][v], ss2);
+        }
+        if constexpr (V == 4) *(float4*)(x + row0 + i) = make_float4(res[e][0], res[e][1], res[e][2], res[e][3]);
+        else x[row0 + i] = res[e][0];
+      }
+    }
+  } else {
+    for (int i = threadIdx.x; i < width; i += RS_THREADS) {
+      const float g = (offset + rv_load_w(w_post, w_post_f32, i)) * (scale ? rv_load_w(scale, scale_f32, i) : 1.0f);
+      const float r = x[row0 + i] + rs_branch<T>(branch, slices, slice_stride, row0 + i) * inv * g;
+      x[row0 + i] = r;
+      ss2 = fmaf(r, r, ss2);
+    }
   }
   if (next == nullptr) return;
   ss2 = rv_block_sum(ss2, scratch);
   const float inv2 = 1.0f / sqrtf(ss2 / (float)width + eps_next);
-  // every thread reads back what it wrote itself
-  for (int i = threadIdx.x; i < width; i += RS_THREADS)
-    next[row0 + i] = rv_from_float<T>(x[row0 + i] * inv2 * (offset_next + rv_load_w(w_next, w_next_f32, i)));
+  if constexpr (E > 0) {
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+      const int i = (e * RS_THREADS + threadIdx.x) * V;
+      if (i < width) {
+#pragma unroll
+        for (int v = 0; v < V; ++v)
+          next[row0 + i + v] = rv_from_float<T>(res[e][v] * inv2 * (offset_next + rv_load_w(w_next, w_next_f32, i + v)));
+      }
+    }
+  } else {
+    // every thread reads back what it wrote itself
+    for (int i = threadIdx.x; i < width; i += RS_THREADS)
+      next[row0 + i] = rv_from_float<T>(x[row0 + i] * inv2 * (offset_next + rv_load_w(w_next, w_next_f32, i)));
+  }
 }
 
 // branch: `dtype` values [rows, width] (slices 0) or 32-bit partial sums [slices][rows][width]; x: float, in place;
@@ -98,13 +189,27 @@ extern "C" int rv_add_rmsnorm_scaled(hipStream_t stream, const void* branch, int
   RV_CHECK(slices >= 0 && (slices == 0 || slice_stride >= (long long)rows * width), "add_rmsnorm_scaled: bad partial sums");
   if (rows == 0) return 0;
   dim3 grid(rows), block(RS_THREADS);
-#define RV_AS(T)                                                                                                      \
-  add_rmsnorm_scaled_kernel<T><<<grid, block, 0, stream>>>(branch, slices, slice_stride, w_post, w_post_f32, scale,   \
-                                                           scale_f32, x, w_next, w_next_f32, (T*)next, width, eps,    \
-                                                           offset, eps_next, offset_next)
-  if (dtype == RV_F32) RV_AS(float);
-  else if (dtype == RV_BF16) RV_AS(bf16_t);
+  // four values a thread and turn where rows, slices and streams all start on 16-byte boundaries
+  const bool vec = width % 4 == 0 && slice_stride % 4 == 0 && (((uintptr_t)x | (uintptr_t)branch) & 15) == 0;
+#define RV_AS(T, E, V)                                                                                                  \
+  add_rmsnorm_scaled_kernel<T, E, V><<<grid, block, 0, stream>>>(branch, slices, slice_stride, w_post, w_post_f32,      \
+                                                                 scale, scale_f32, x, w_next, w_next_f32, (T*)next,     \
+                                                                 width, eps, offset, eps_next, offset_next)
+#define RV_AS_T(T)                                                 \
+  do {                                                             \
+    const int e_ = rv_div_up(width, RS_THREADS * (vec ? 4 : 1));   \
+    if (vec && e_ <= 1) RV_AS(T, 1, 4);                            \
+    else if (vec && e_ <= 2) RV_AS(T, 2, 4);                       \
+    else if (vec && e_ <= 4) RV_AS(T, 4, 4);                       \
+    else if (vec && e_ <= 8) RV_AS(T, 8, 4);                       \
+    else if (!vec && e_ <= 2) RV_AS(T, 2, 1);                      \
+    else if (!vec && e_ <= 8) RV_AS(T, 8, 1);                      \
+    else RV_AS(T, 0, 1);                                           \
+  } while (0)
+  if (dtype == RV_F32) RV_AS_T(float);
+  else if (dtype == RV_BF16) RV_AS_T(bf16_t);
   else return rv_fail("add_rmsnorm_scaled: unsupported dtype %d", dtype);
+#undef RV_AS_T
 #undef RV_AS
   RV_LAUNCH_CHECK("add_rmsnorm_scaled");
   return 0;

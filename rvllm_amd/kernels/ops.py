@@ -1575,8 +1575,8 @@ def delta_rule(qkv: torch.Tensor, q_off: int, k_off: int, v_off: int, ab: torch.
     """The gated delta rule over the step's tokens, request by request in order.  ``qkv`` float32 rows: unit
     queries (scaled) and keys of ``kv_heads`` heads of ``dk``, values of ``heads`` heads of ``dv``, at their
     offsets; ``ab`` rows hold the decay's input of head h at ``a_col + h`` and beta's at ``b_col + h``;
-    g = exp(-exp(A_log) softplus(a + dt_bias)), beta = sigmoid(b).  Per head S [dk, dv] (32-bit, in the
-    request's slot from ``state_off``): S <- g S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q.  Returns o as
+    g = exp(-exp(A_log) softplus(a + dt_bias)), beta = sigmoid(b).  Per head S (32-bit, in the request's
+    slot from ``state_off``, stored ``[heads, dv, dk]``: a column's dk numbers side by side): S <- g S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q.  Returns o as
     float32 ``[tokens, heads * dv]``."""
     _gpu(qkv, A_log, dt_bias)
     n = qkv.shape[0]
@@ -1595,7 +1595,7 @@ def delta_rule(qkv: torch.Tensor, q_off: int, k_off: int, v_off: int, ab: torch.
         _stream(), _ptr(qkv), _c_ll(qkv.stride(0)), _c_int(q_off), _c_int(k_off), _c_int(v_off), _ptr(ab), _dt(ab),
         _c_ll(ab.stride(0)), _c_int(a_col), _c_int(b_col), _ptr(A_log), _ptr(dt_bias), _ptr(slots), _c_ll(stride),
         _c_ll(state_off), _ptr(step.q_start), _ptr(step.state_slot), _ptr(out), _c_int(step.num_requests), _c_int(heads),
-        _c_int(kv_heads), _c_int(dk), _c_int(dv)))
+        _c_int(kv_heads), _c_int(dk), _c_int(dv), _c_int(step.max_portion)))
     return out
 
 
@@ -1642,5 +1642,5 @@ def selective_scan(x: torch.Tensor, z: torch.Tensor, z_col0: int, dt: torch.Tens
         _stream(), _ptr(x), _c_ll(x.stride(0)), z.data_ptr() + z_col0 * z.element_size(), _c_ll(z.stride(0)), _ptr(dt),
         _c_ll(dt.stride(0)), _ptr(dt_bias), _ptr(bc), _c_ll(bc.stride(0)), _c_int(b_col), _c_int(c_col), _ptr(A_log),
         _ptr(D), _ptr(slots), _c_ll(stride), _c_ll(state_off), _ptr(step.q_start), _ptr(step.state_slot), _ptr(out),
-        _dt(x), _c_int(step.num_requests), _c_int(channels), _c_int(n_state)))
+        _dt(x), _c_int(step.num_requests), _c_int(channels), _c_int(n_state), _c_int(step.max_portion)))
     return out

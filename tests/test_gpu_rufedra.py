@@ -137,7 +137,7 @@ def test_delta_rule_whole_and_cut_give_the_same_bits(dtype, heads, kv_heads, dk,
                                        heads, kv_heads, dk, dv).cpu())
         results.append(torch.cat(rows))
         close(results[-1], want, torch.float32, f"cut {sizes}", f32=1e-4)
-        close(slots[2, 5:].view(heads, dk, dv), torch.stack(last), torch.float32, "the state", f32=1e-4)
+        close(slots[2, 5:].view(heads, dv, dk).transpose(1, 2), torch.stack(last), torch.float32, "the state", f32=1e-4)
         assert float(slots[:2].abs().max()) == 0.0 and float(slots[2, :5].abs().max()) == 0.0
     assert torch.equal(results[0], results[1]) and torch.equal(results[0], results[2])
 
