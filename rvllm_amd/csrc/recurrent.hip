@@ -60,15 +60,18 @@ __device__ __forceinline__ float rec_decay_exp<bf16_t>(float x) {
 // position first - (taps - 1) + s); a fresh slot's zeros are the zeros before the start of a sequence.
 // A wave takes a group of `group` channels of one token; with unit_eps >= 0 the group's outputs are divided by
 // sqrt(sum y^2 + unit_eps) and the first `scaled_groups` groups multiplied by `group_scale`.
+// `move_state`: every request of the step brings exactly one token (the host knows), so the lane that works on a
+// channel is the only one that reads that channel's state rows, and moves them on itself (a row up, the token's
+// input last) instead of leaving that to conv_state_update.
 // ---------------------------------------------------------------------------
 template <typename T, typename TO>
 __global__ void __launch_bounds__(256)
 causal_conv_kernel(const T* __restrict__ in, long long ld_in, const float* __restrict__ w, const float* __restrict__ bias,
-                   int taps, const float* __restrict__ state, long long slot_stride, long long state_off,
+                   int taps, float* __restrict__ state, long long slot_stride, long long state_off,
                    int state_ld, const int* __restrict__ positions, const int* __restrict__ token_req,
                    const int* __restrict__ q_start, const int* __restrict__ chunk_start,
                    const int* __restrict__ state_slot, TO* __restrict__ out, long long ld_out, int channels, int group,
-                   int groups, int num_tokens, float unit_eps, int scaled_groups, float group_scale) {
+                   int groups, int num_tokens, float unit_eps, int scaled_groups, float group_scale, int move_state) {
   const int lane = threadIdx.x & (RV_WAVE - 1);
   const long long unit = (long long)blockIdx.x * (blockDim.x / RV_WAVE) + threadIdx.x / RV_WAVE;
   if (unit >= (long long)num_tokens * groups) return;  // the whole wave
@@ -78,7 +81,7 @@ causal_conv_kernel(const T* __restrict__ in, long long ld_in, const float* __res
   const int first_pos = chunk_start[req];
   const int first_tok = q_start[req];
   const int rel = positions[t] - first_pos;  // place of the token in its portion
-  const float* st = state + (long long)state_slot[req] * slot_stride + state_off;
+  float* st = state + (long long)state_slot[req] * slot_stride + state_off;
   float ss = 0.f;
   for (int c0 = 0; c0 < group; c0 += RV_WAVE) {  // (two passes when the group is normed: the sum, then the store)
     const int c = grp * group + c0 + lane;
@@ -91,7 +94,13 @@ causal_conv_kernel(const T* __restrict__ in, long long ld_in, const float* __res
         acc = fmaf(w[(long long)c * taps + j], x, acc);
       }
       const float y = rv_round_to<T>(rec_silu(acc));
-      if (unit_eps < 0.f) out[(long long)t * ld_out + c] = rv_from_float<TO>(y);
+      if (unit_eps < 0.f) {
+        out[(long long)t * ld_out + c] = rv_from_float<TO>(y);
+        if (move_state) {  // rel is 0: rows 1 .. taps - 2 move up, the token's input goes last
+          for (int s_ = 0; s_ + 2 < taps; ++s_) st[(long long)s_ * state_ld + c] = st[(long long)(s_ + 1) * state_ld + c];
+          if (taps > 1) st[(long long)(taps - 2) * state_ld + c] = rv_to_float(in[(long long)first_tok * ld_in + c]);
+        }
+      }
       ss = fmaf(y, y, ss);
     }
   }
@@ -109,6 +118,10 @@ causal_conv_kernel(const T* __restrict__ in, long long ld_in, const float* __res
         acc = fmaf(w[(long long)c * taps + j], x, acc);
       }
       out[(long long)t * ld_out + c] = rv_from_float<TO>(rv_round_to<T>(rec_silu(acc)) * mult);
+      if (move_state) {
+        for (int s_ = 0; s_ + 2 < taps; ++s_) st[(long long)s_ * state_ld + c] = st[(long long)(s_ + 1) * state_ld + c];
+        if (taps > 1) st[(long long)(taps - 2) * state_ld + c] = rv_to_float(in[(long long)first_tok * ld_in + c]);
+      }
     }
   }
 }
@@ -117,11 +130,11 @@ causal_conv_kernel(const T* __restrict__ in, long long ld_in, const float* __res
 // float [channels] or null.  state: float, row s of a slot's block at state_off + s * state_ld.  out: float
 // (out_f32) or `dtype`.  unit_eps < 0: no unit length.
 extern "C" int rv_causal_conv(hipStream_t stream, const void* in, int dtype, long long ld_in, const float* w,
-                              const float* bias, int taps, const float* state, long long slot_stride,
+                              const float* bias, int taps, float* state, long long slot_stride,
                               long long state_off, int state_ld, const int* positions, const int* token_req,
                               const int* q_start, const int* chunk_start, const int* state_slot, void* out,
                               int out_f32, long long ld_out, int channels, int group, int num_tokens, float unit_eps,
-                              int scaled_groups, float group_scale) {
+                              int scaled_groups, float group_scale, int move_state) {
   RV_CHECK(in && w && state && positions && token_req && q_start && chunk_start && state_slot && out,
            "causal_conv: null argument");
   RV_CHECK(taps >= 1 && taps <= REC_MAX_TAPS && channels > 0 && group > 0 && num_tokens >= 0 && state_ld >= channels,
@@ -134,7 +147,8 @@ extern "C" int rv_causal_conv(hipStream_t stream, const void* in, int dtype, lon
   causal_conv_kernel<T, TO><<<grid, block, 0, stream>>>((const T*)in, ld_in, w, bias, taps, state, slot_stride,      \
                                                         state_off, state_ld, positions, token_req, q_start,          \
                                                         chunk_start, state_slot, (TO*)out, ld_out, channels, group,  \
-                                                        groups, num_tokens, unit_eps, scaled_groups, group_scale)
+                                                        groups, num_tokens, unit_eps, scaled_groups, group_scale,     \
+                                                        move_state)
   if (dtype == RV_F32) RV_CC(float, float);
   else if (dtype == RV_BF16 && out_f32) RV_CC(bf16_t, float);
   else if (dtype == RV_BF16) RV_CC(bf16_t, bf16_t);

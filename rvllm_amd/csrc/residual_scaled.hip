@@ -2,6 +2,7 @@
 //
 //   rmsnorm_cast         y = x / sqrt(mean(x^2) + eps) * (offset + w)          x of one type, y of another
 //   add_rmsnorm_scaled   x <- x + branch / sqrt(mean(branch^2) + eps) * (offset + w_post) * scale
+//                        (branch may be wa * branch + wb * branch2: two mixers side by side, each with its weight)
 //                        next = x / sqrt(mean(x^2) + eps_next) * (offset_next + w_next)   optionally
 //
 // x is float whatever the activations' type T; the branch is stored as T or given as unreduced 32-bit partial sums
@@ -85,6 +86,7 @@ __device__ __forceinline__ void rs_load_branch(const void* p, bool sliced, size_
 template <typename T, int E, int V>
 __global__ void __launch_bounds__(RS_THREADS)
 add_rmsnorm_scaled_kernel(const void* __restrict__ branch, int slices, long long slice_stride,
+                          const void* __restrict__ branch2, int slices2, long long slice_stride2, float wa, float wb,
                           const void* __restrict__ w_post, int w_post_f32, const void* __restrict__ scale,
                           int scale_f32, float* __restrict__ x, const void* __restrict__ w_next, int w_next_f32,
                           T* __restrict__ next, int width, float eps, float offset, float eps_next,
@@ -122,13 +124,40 @@ add_rmsnorm_scaled_kernel(const void* __restrict__ branch, int slices, long long
 #pragma unroll
         for (int v = 0; v < V; ++v) val[e][v] += part[e][v];
     }
+    if (branch2 != nullptr) {
+      float other[E][V];
+#pragma unroll
+      for (int e = 0; e < E; ++e)
+#pragma unroll
+        for (int v = 0; v < V; ++v) other[e][v] = 0.f;
+      const int rounds2 = slices2 > 0 ? slices2 : 1;
+      for (int s = 0; s < rounds2; ++s) {
+        float part[E][V];
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+          const int i = (e * RS_THREADS + threadIdx.x) * V;
+#pragma unroll
+          for (int v = 0; v < V; ++v) part[e][v] = 0.f;
+          if (i < width) rs_load_branch<T, V>(branch2, slices2 > 0, (size_t)s * slice_stride2 + row0 + i, part[e]);
+        }
+#pragma unroll
+        for (int e = 0; e < E; ++e)
+#pragma unroll
+          for (int v = 0; v < V; ++v) other[e][v] += part[e][v];
+      }
+#pragma unroll
+      for (int e = 0; e < E; ++e)
+#pragma unroll
+        for (int v = 0; v < V; ++v) val[e][v] = wa * val[e][v] + wb * other[e][v];
+    }
 #pragma unroll
     for (int e = 0; e < E; ++e)
 #pragma unroll
       for (int v = 0; v < V; ++v) ss = fmaf(val[e][v], val[e][v], ss);
   } else {
     for (int i = threadIdx.x; i < width; i += RS_THREADS) {
-      const float v = rs_branch<T>(branch, slices, slice_stride, row0 + i);
+      float v = rs_branch<T>(branch, slices, slice_stride, row0 + i);
+      if (branch2 != nullptr) v = wa * v + wb * rs_branch<T>(branch2, slices2, slice_stride2, row0 + i);
       ss = fmaf(v, v, ss);
     }
   }
@@ -152,7 +181,9 @@ add_rmsnorm_scaled_kernel(const void* __restrict__ branch, int slices, long long
   } else {
     for (int i = threadIdx.x; i < width; i += RS_THREADS) {
       const float g = (offset + rv_load_w(w_post, w_post_f32, i)) * (scale ? rv_load_w(scale, scale_f32, i) : 1.0f);
-      const float r = x[row0 + i] + rs_branch<T>(branch, slices, slice_stride, row0 + i) * inv * g;
+      float v = rs_branch<T>(branch, slices, slice_stride, row0 + i);
+      if (branch2 != nullptr) v = wa * v + wb * rs_branch<T>(branch2, slices2, slice_stride2, row0 + i);
+      const float r = x[row0 + i] + v * inv * g;
       x[row0 + i] = r;
       ss2 = fmaf(r, r, ss2);
     }
@@ -177,9 +208,10 @@ add_rmsnorm_scaled_kernel(const void* __restrict__ branch, int slices, long long
   }
 }
 
-// branch: `dtype` values [rows, width] (slices 0) or 32-bit partial sums [slices][rows][width]; x: float, in place;
-// next: `dtype`, with w_next, or both null.
+// branch: `dtype` values [rows, width] (slices 0) or 32-bit partial sums [slices][rows][width]; branch2: the same or
+// null; x: float, in place; next: `dtype`, with w_next, or both null.
 extern "C" int rv_add_rmsnorm_scaled(hipStream_t stream, const void* branch, int slices, long long slice_stride,
+                                     const void* branch2, int slices2, long long slice_stride2, float wa, float wb,
                                      const void* w_post, int w_post_f32, const void* scale, int scale_f32, float* x,
                                      const void* w_next, int w_next_f32, void* next, int dtype, int rows, int width,
                                      float eps, float offset, float eps_next, float offset_next) {
@@ -187,12 +219,16 @@ extern "C" int rv_add_rmsnorm_scaled(hipStream_t stream, const void* branch, int
            width);
   RV_CHECK((w_next == nullptr) == (next == nullptr), "add_rmsnorm_scaled: the next norm needs both weight and output");
   RV_CHECK(slices >= 0 && (slices == 0 || slice_stride >= (long long)rows * width), "add_rmsnorm_scaled: bad partial sums");
+  RV_CHECK(slices2 >= 0 && (slices2 == 0 || slice_stride2 >= (long long)rows * width),
+           "add_rmsnorm_scaled: bad partial sums of the second branch");
   if (rows == 0) return 0;
   dim3 grid(rows), block(RS_THREADS);
   // four values a thread and turn where rows, slices and streams all start on 16-byte boundaries
-  const bool vec = width % 4 == 0 && slice_stride % 4 == 0 && (((uintptr_t)x | (uintptr_t)branch) & 15) == 0;
+  const bool vec = width % 4 == 0 && slice_stride % 4 == 0 && slice_stride2 % 4 == 0 &&
+                   (((uintptr_t)x | (uintptr_t)branch | (uintptr_t)branch2) & 15) == 0;
 #define RV_AS(T, E, V)                                                                                                  \
-  add_rmsnorm_scaled_kernel<T, E, V><<<grid, block, 0, stream>>>(branch, slices, slice_stride, w_post, w_post_f32,      \
+  add_rmsnorm_scaled_kernel<T, E, V><<<grid, block, 0, stream>>>(branch, slices, slice_stride, branch2, slices2,        \
+                                                                 slice_stride2, wa, wb, w_post, w_post_f32,             \
                                                                  scale, scale_f32, x, w_next, w_next_f32, (T*)next,     \
                                                                  width, eps, offset, eps_next, offset_next)
 #define RV_AS_T(T)                                                 \

@@ -9,6 +9,9 @@
 //   write     queries to q_out [tokens, nq * hd]; keys (rotated, normed) and values into the paged cache of
 //             kv_layout.h at the token's position; a negative page skips the write.  v_col < 0: the value is the
 //             key as it came in, before rotation and norm.
+//   bias      null, or one 32-bit number for every column of a row of `in`: the projections' biases, added as the
+//             row is read (to queries, keys and values alike; the sum is rounded to the activations' type, as a
+//             projection with its bias would have been stored)
 // All arithmetic is 32-bit; rows of `in` are ld apart and hold the queries from q_col and the keys from k_col on.
 #include "common.h"
 #include "kv_layout.h"
@@ -19,7 +22,7 @@
 template <typename T>
 __global__ void __launch_bounds__(256)
 rotate_norm_write_kernel(const T* __restrict__ in, long long ld, int q_col, int k_col, int v_col,
-                         T* __restrict__ q_out, const void* __restrict__ q_w, const void* __restrict__ k_w, int w_f32,
+                         const float* __restrict__ bias, T* __restrict__ q_out, const void* __restrict__ q_w, const void* __restrict__ k_w, int w_f32,
                          float eps, float offset, int norm_mode, const float* __restrict__ cos_t,
                          const float* __restrict__ sin_t, int rot, const int* __restrict__ positions,
                          const int* __restrict__ token_req, const int* __restrict__ table, int table_width,
@@ -34,7 +37,9 @@ rotate_norm_write_kernel(const T* __restrict__ in, long long ld, int q_col, int 
   const bool is_q = head < nq;
   if (!is_q && !write_kv) return;
   const int kvh = head - nq;
-  const T* src = in + (long long)t * ld + (is_q ? q_col + head * hd : k_col + kvh * hd);
+  const int col0 = is_q ? q_col + head * hd : k_col + kvh * hd;
+  const T* src = in + (long long)t * ld + col0;
+  const float* b = bias ? bias + col0 : nullptr;
   const void* w = is_q ? q_w : k_w;
   const int half = rot / 2;
   float raw[RNW_E], val[RNW_E];
@@ -42,7 +47,7 @@ rotate_norm_write_kernel(const T* __restrict__ in, long long ld, int q_col, int 
 #pragma unroll
   for (int e = 0; e < RNW_E; ++e) {
     const int d = e * RV_WAVE + lane;
-    raw[e] = d < hd ? rv_to_float(src[d]) : 0.f;
+    raw[e] = d < hd ? (b ? rv_round_to<T>(rv_to_float(src[d]) + b[d]) : rv_to_float(src[d])) : 0.f;
     ss_raw = fmaf(raw[e], raw[e], ss_raw);
   }
   float inv_before = 1.0f;
@@ -55,7 +60,7 @@ rotate_norm_write_kernel(const T* __restrict__ in, long long ld, int q_col, int 
     if (norm_mode == 1 && d < hd) x *= inv_before * (w ? offset + rv_load_w(w, w_f32, d) : 1.0f);
     if (d < rot) {
       const int partner = d < half ? d + half : d - half;
-      float y = rv_to_float(src[partner]);
+      float y = b ? rv_round_to<T>(rv_to_float(src[partner]) + b[partner]) : rv_to_float(src[partner]);
       if (norm_mode == 1) y *= inv_before * (w ? offset + rv_load_w(w, w_f32, partner) : 1.0f);
       const int i = d < half ? d : d - half;
       const float c = cos_t[(long long)t * half + i], s = sin_t[(long long)t * half + i];
@@ -86,18 +91,20 @@ rotate_norm_write_kernel(const T* __restrict__ in, long long ld, int q_col, int 
   if (page < 0 || page >= num_pages) return;
   const int slot = pos % page_size;
   const T* vsrc = v_col >= 0 ? in + (long long)t * ld + v_col + kvh * hd : nullptr;
+  const float* vb = (bias && v_col >= 0) ? bias + v_col + kvh * hd : nullptr;
 #pragma unroll
   for (int e = 0; e < RNW_E; ++e) {
     const int d = e * RV_WAVE + lane;
     if (d < hd) {
       k_pages[rv_k_index(page, kvh, slot, d, nkv, page_size, hd)] = rv_from_float<T>(val[e]);
-      v_pages[rv_v_index(page, kvh, slot, d, nkv, page_size, hd)] = vsrc ? vsrc[d] : rv_from_float<T>(raw[e]);
+      v_pages[rv_v_index(page, kvh, slot, d, nkv, page_size, hd)] =
+          vsrc ? (vb ? rv_from_float<T>(rv_to_float(vsrc[d]) + vb[d]) : vsrc[d]) : rv_from_float<T>(raw[e]);
     }
   }
 }
 
 extern "C" int rv_rotate_norm_write(hipStream_t stream, const void* in, long long ld, int q_col, int k_col, int v_col,
-                                    void* q_out, const void* q_w, const void* k_w, int w_f32, float eps, float offset,
+                                    const float* bias, void* q_out, const void* q_w, const void* k_w, int w_f32, float eps, float offset,
                                     int norm_mode, const float* cos_t, const float* sin_t, int rot,
                                     const int* positions, const int* token_req, const int* table, int table_width,
                                     void* k_pages, void* v_pages, int page_size, int num_pages, int dtype,
@@ -114,7 +121,7 @@ extern "C" int rv_rotate_norm_write(hipStream_t stream, const void* in, long lon
   const long long units = (long long)num_tokens * (nq + nkv);
   dim3 grid(rv_div_up(units, 4)), block(256);
 #define RV_RNW(T)                                                                                                    \
-  rotate_norm_write_kernel<T><<<grid, block, 0, stream>>>((const T*)in, ld, q_col, k_col, v_col, (T*)q_out, q_w, k_w, \
+  rotate_norm_write_kernel<T><<<grid, block, 0, stream>>>((const T*)in, ld, q_col, k_col, v_col, bias, (T*)q_out, q_w, k_w, \
                                                           w_f32, eps, offset, norm_mode, cos_t, sin_t, rot, positions, \
                                                           token_req, table, table_width, (T*)k_pages, (T*)v_pages,     \
                                                           page_size, num_pages, num_tokens, nq, nkv, hd, write_kv)

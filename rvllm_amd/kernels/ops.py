@@ -177,7 +177,7 @@ class TiledWeight:
 
 def as_tensor(x) -> torch.Tensor:
     """A plain tensor from a tensor or from unreduced ``SlicedSums``."""
-    return x.as_tensor() if isinstance(x, SlicedSums) else x
+    return x.as_tensor() if isinstance(x, (SlicedSums, BranchSum)) else x
 
 
 def _branch_args(x, what: str):
@@ -1395,13 +1395,34 @@ def rmsnorm_cast(x: torch.Tensor, weight: torch.Tensor, eps: float, offset: floa
     return out
 
 
+class BranchSum:
+    """a * x + b * y for two branches of one shape and type (tensors or unreduced ``SlicedSums``), not added up yet:
+    the kernel that norms a branch and adds it to the residual stream takes the two as they are
+    (``add_rmsnorm_scaled``); anything else calls ``as_tensor``."""
+
+    def __init__(self, x, y, a: float, b: float):
+        self.x, self.y, self.a, self.b = x, y, float(a), float(b)
+        self.shape, self.device = x.shape, x.device
+        self.dtype = x.dtype
+
+    def as_tensor(self) -> torch.Tensor:
+        return weighted_sum(self.x, self.y, self.a, self.b).as_tensor()
+
+
 def add_rmsnorm_scaled(branch, weight: torch.Tensor, eps: float, offset: float, scale: Optional[torch.Tensor],
                        residual: torch.Tensor, next_weight: Optional[torch.Tensor] = None, next_eps: float = 0.0,
                        next_offset: float = 0.0) -> Optional[torch.Tensor]:
     """residual += rmsnorm(branch) * scale on a 32-bit ``residual``; ``scale`` is one number a channel or None.
     With ``next_weight`` also returns rmsnorm(residual) in the branch's type.  ``branch`` is a tensor of the
-    activations' type or ``SlicedSums``."""
+    activations' type, ``SlicedSums``, or a ``BranchSum`` of two of these."""
+    second, wa, wb = None, 1.0, 0.0
+    if isinstance(branch, BranchSum):
+        branch, second, wa, wb = branch.x, branch.y, branch.a, branch.b
     bptr, slices, stride, rows, width, bdtype = _branch_args(branch, "add_rmsnorm_scaled")
+    sptr, s_slices, s_stride = None, 0, 0
+    if second is not None:
+        sptr, s_slices, s_stride, s_rows, s_width, s_dtype = _branch_args(second, "add_rmsnorm_scaled")
+        _need((s_rows, s_width, s_dtype) == (rows, width, bdtype), "add_rmsnorm_scaled: two branches of one shape and type")
     _gpu(weight, scale, residual, next_weight)
     _need(residual.shape == (rows, width) and residual.dtype == torch.float32,
           "add_rmsnorm_scaled: the residual stream is a 32-bit matrix of the branch's shape")
@@ -1412,7 +1433,8 @@ def add_rmsnorm_scaled(branch, weight: torch.Tensor, eps: float, offset: float, 
         _need(next_weight.shape == (width,) and next_weight.dtype in _DT, "add_rmsnorm_scaled: bad next weight")
         nxt = torch.empty((rows, width), dtype=bdtype, device=residual.device)
     _check(library().rv_add_rmsnorm_scaled(
-        _stream(), bptr, _c_int(slices), _c_ll(stride), _ptr(weight), _c_int(weight.dtype == torch.float32),
+        _stream(), bptr, _c_int(slices), _c_ll(stride), sptr, _c_int(s_slices), _c_ll(s_stride), _c_float(wa),
+        _c_float(wb), _ptr(weight), _c_int(weight.dtype == torch.float32),
         _ptr(scale), _c_int(scale is not None and scale.dtype == torch.float32), _ptr(residual), _ptr(next_weight),
         _c_int(next_weight is not None and next_weight.dtype == torch.float32), _ptr(nxt), _DT[bdtype], _c_int(rows),
         _c_int(width), _c_float(eps), _c_float(offset), _c_float(next_eps), _c_float(next_offset)))
@@ -1449,13 +1471,17 @@ def rotate_norm_write(proj: torch.Tensor, q_col: int, k_col: int, v_col: Optiona
                       norm_mode: int, rope: Optional[tuple[torch.Tensor, torch.Tensor]], rotary_dim: int,
                       positions: torch.Tensor, token_req: torch.Tensor, block_table: Optional[torch.Tensor],
                       k_pages: Optional[torch.Tensor], v_pages: Optional[torch.Tensor], num_q_heads: int,
-                      num_kv_heads: int, head_dim: int, write_kv: bool = True) -> torch.Tensor:
+                      num_kv_heads: int, head_dim: int, write_kv: bool = True,
+                      bias: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Queries and keys from the rows of ``proj`` (queries from column ``q_col``, keys from ``k_col``, values from
     ``v_col`` or, with None, the keys as they stand there): rotation of the first ``rotary_dim`` dimensions of a
     head, dimension i paired with i + rotary_dim / 2; per-head RMS norm before or after it (``norm_mode``), with
-    the weights or without; queries to ``q_out``, keys and values into the cache."""
+    the weights or without; queries to ``q_out``, keys and values into the cache.  ``bias``: one 32-bit number
+    for every column of ``proj``, added to queries, keys and values as they are read."""
     cos, sin = rope if rope is not None else (None, None)
-    _gpu(q_out, q_weight, k_weight, cos, sin, positions, token_req, block_table, k_pages, v_pages)
+    _gpu(q_out, q_weight, k_weight, cos, sin, positions, token_req, block_table, k_pages, v_pages, bias)
+    _need(bias is None or (bias.dtype == torch.float32 and bias.shape == (proj.shape[1],)),
+          "rotate_norm_write: the bias holds a 32-bit number for every column of the rows")
     _need(proj.is_cuda and proj.dim() == 2 and proj.stride(1) == 1, "rotate_norm_write: rows of projections expected")
     _i32(positions, token_req)
     n = proj.shape[0]
@@ -1486,7 +1512,7 @@ def rotate_norm_write(proj: torch.Tensor, q_col: int, k_col: int, v_col: Optiona
         width = block_table.shape[1]
     _check(library().rv_rotate_norm_write(
         _stream(), _ptr(proj), _c_ll(proj.stride(0)), _c_int(q_col), _c_int(k_col), _c_int(-1 if v_col is None else v_col),
-        _ptr(q_out), _ptr(q_weight), _ptr(k_weight), _c_int(w_f32), _c_float(eps), _c_float(offset), _c_int(norm_mode),
+        _ptr(bias), _ptr(q_out), _ptr(q_weight), _ptr(k_weight), _c_int(w_f32), _c_float(eps), _c_float(offset), _c_int(norm_mode),
         _ptr(cos), _ptr(sin), _c_int(rot), _ptr(positions), _ptr(token_req), _ptr(block_table), _c_int(width),
         _ptr(k_pages), _ptr(v_pages), _c_int(page_size), _c_int(num_pages), _dt(proj), _c_int(n), _c_int(num_q_heads),
         _c_int(num_kv_heads), _c_int(head_dim), _c_int(int(write_kv))))
@@ -1519,7 +1545,7 @@ def _state_args(slots: torch.Tensor, what: str) -> int:
 def causal_conv(x: torch.Tensor, col0: int, channels: int, weight: torch.Tensor, bias: Optional[torch.Tensor],
                 slots: torch.Tensor, state_off: int, step, out: torch.Tensor, out_col0: int = 0, group: int = 64,
                 unit_eps: Optional[float] = None, scaled_groups: int = 0, group_scale: float = 1.0,
-                state_ld: Optional[int] = None) -> torch.Tensor:
+                state_ld: Optional[int] = None, move_state: bool = False) -> torch.Tensor:
     """Short causal convolution over time and silu for the channels ``col0 .. col0 + channels`` of the rows of
     ``x``: ``weight`` is float32 ``[channels, taps]`` (the last tap is the token's own), ``bias`` float32 or None.
     The inputs before a request's first token of the step come from its state slot (``taps - 1`` rows of
@@ -1527,8 +1553,11 @@ def causal_conv(x: torch.Tensor, col0: int, channels: int, weight: torch.Tensor,
     Results go to the columns ``out_col0 ...`` of ``out`` (float32 or the type of ``x``).  With ``unit_eps`` every
     group of ``group`` channels is divided by sqrt(sum of squares + unit_eps), and the first ``scaled_groups``
     groups are multiplied by ``group_scale``.  ``state_ld``: the channels a row of the state holds, when these
-    are a part of them (``state_off`` then points at this part's first channel)."""
+    are a part of them (``state_off`` then points at this part's first channel).  ``move_state``: the kernel also
+    moves the state on for these channels; only for a step in which every request brings exactly one token (see
+    ``conv_moves_state``), where it replaces ``conv_state_update``."""
     _gpu(weight, bias)
+    _need(not move_state or step.max_portion == 1, "causal_conv: the state moves with the kernel in steps of single tokens only")
     state_ld = channels if state_ld is None else int(state_ld)
     _need(x.is_cuda and x.dim() == 2 and x.stride(1) == 1 and out.is_cuda and out.dim() == 2 and out.stride(1) == 1,
           "causal_conv: rows expected")
@@ -1551,8 +1580,14 @@ def causal_conv(x: torch.Tensor, col0: int, channels: int, weight: torch.Tensor,
         _ptr(step.token_req), _ptr(step.q_start), _ptr(step.chunk_start), _ptr(step.state_slot),
         out.data_ptr() + out_col0 * out.element_size(), _c_int(out.dtype == torch.float32 and x.dtype != torch.float32),
         _c_ll(out.stride(0)), _c_int(channels), _c_int(group), _c_int(n),
-        _c_float(-1.0 if unit_eps is None else unit_eps), _c_int(scaled_groups), _c_float(group_scale)))
+        _c_float(-1.0 if unit_eps is None else unit_eps), _c_int(scaled_groups), _c_float(group_scale),
+        _c_int(int(move_state))))
     return out
+
+
+def conv_moves_state(step) -> bool:
+    """Whether ``causal_conv`` may move the convolutions' state on itself in this step: every request brings one token."""
+    return step.max_portion == 1
 
 
 def conv_state_update(x: torch.Tensor, col0: int, channels: int, taps: int, slots: torch.Tensor, state_off: int,

@@ -166,8 +166,9 @@ class PagedAttention(Mixer):
         """The variants: the rows of the fused projection hold q | k | (v) | (g)."""
         n = x.shape[0]
         proj = linear(x, self.w_qkv)
-        if self.b_qkv is not None:
-            proj = ops.add_bias(proj, self.b_qkv)
+        bias = self.b_qkv
+        if bias is not None and "g" in self.bias:  # the gate reads its columns from the rows: its bias goes in there
+            proj, bias = ops.add_bias(proj, bias), None
         q = torch.empty((n, self.q_size), dtype=x.dtype, device=x.device)
         table = step.block_tables[cache.group]
         norm = self.qk_norm or {}
@@ -179,7 +180,7 @@ class PagedAttention(Mixer):
             proj, 0, k_col, v_col, q, self.q_norm_w, self.k_norm_w, float(norm.get("eps", 0.0)),
             1.0 if norm.get("unit_offset", False) else 0.0, mode, self.position.tables(step),
             self.position.rotary_dim, step.positions, step.token_req, table, cache.k_pages, cache.v_pages,
-            self.num_heads, self.num_kv_heads, self.head_dim, write_kv=cache.writes)
+            self.num_heads, self.num_kv_heads, self.head_dim, write_kv=cache.writes, bias=bias)
         attn = torch.empty_like(q)
         ops.paged_attention(q, cache.k_pages, cache.v_pages, table, step, attn, self.num_heads, self.scale,
                             self.window)

@@ -107,12 +107,14 @@ class GatedDeltaRule(Mixer):
         proj = linear(x, self.w_in)  # [n, q | k | v | g | b | a]
         qk = 2 * self.qk_size
         qkv = torch.empty((n, self.conv_channels), dtype=torch.float32, device=x.device)
+        moves = ops.conv_moves_state(step)  # single tokens: the convolutions move their state on themselves
         ops.causal_conv(proj, 0, qk, self.conv_qk, None, slots, 0, step, qkv, 0, group=self.dim,
                         unit_eps=self.unit_eps, scaled_groups=self.kv_heads, group_scale=self.dim ** -0.5,
-                        state_ld=self.conv_channels)
+                        state_ld=self.conv_channels, move_state=moves)
         ops.causal_conv(proj, qk, self.v_size, self.conv_v, None, slots, qk, step, qkv, qk,
-                        state_ld=self.conv_channels)
-        ops.conv_state_update(proj, 0, self.conv_channels, self.taps, slots, 0, step)
+                        state_ld=self.conv_channels, move_state=moves)
+        if not moves:
+            ops.conv_state_update(proj, 0, self.conv_channels, self.taps, slots, 0, step)
         o = ops.delta_rule(qkv, 0, self.qk_size, qk, proj, self.a_col, self.b_col, self.A_log, self.dt_bias, slots,
                            self.s_off, step, self.heads, self.kv_heads, self.dim, self.vdim)
         y = ops.head_norm_gate(o, proj, self.g_col, self.norm_w, self.eps, self.heads, self.vdim, x.dtype)

@@ -84,8 +84,10 @@ class SelectiveScan(Mixer):
         I, N, R = self.inner, self.n_state, self.dt_rank
         proj = linear(x, self.w_in)  # [n, x | z]
         xc = torch.empty((n, I), dtype=x.dtype, device=x.device)
-        ops.causal_conv(proj, 0, I, self.conv_w, self.conv_b, slots, 0, step, xc)
-        ops.conv_state_update(proj, 0, I, self.taps, slots, 0, step)
+        moves = ops.conv_moves_state(step)  # single tokens: the convolution moves its state on itself
+        ops.causal_conv(proj, 0, I, self.conv_w, self.conv_b, slots, 0, step, xc, move_state=moves)
+        if not moves:
+            ops.conv_state_update(proj, 0, I, self.taps, slots, 0, step)
         dbc = linear(xc, self.w_x)  # [n, dt | B | C]
         dt = linear(dbc[:, :R], self.w_dt)
         y = ops.selective_scan(xc, proj, I, dt, self.dt_b, dbc, R, R + N, self.A_log, self.D, slots, self.s_off, step)

@@ -41,10 +41,12 @@ class SideBySide(Mixer):
 
     def forward(self, x: torch.Tensor, step, cache) -> torch.Tensor:
         outs = [m.forward(x, step, view) for m, view in zip(self.members, cache)]
+        if len(outs) == 2:  # left to the kernel that norms the sum and adds it to the stream
+            return ops.BranchSum(outs[0], outs[1], self.scales[0], self.scales[1])
         total = ops.weighted_sum(outs[0], outs[1], self.scales[0], self.scales[1])
-        for out, scale in zip(outs[2:], self.scales[2:]):
+        for out, scale in zip(outs[2:-1], self.scales[2:-1]):
             total = ops.weighted_sum(total, out, 1.0, scale)
-        return total
+        return ops.BranchSum(total, outs[-1], 1.0, self.scales[-1])
 
 
 MIXERS.register("side_by_side", SideBySide)

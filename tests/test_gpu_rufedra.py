@@ -63,7 +63,7 @@ def test_convolution_with_its_state_under_any_cutting(dtype, taps, channels, gro
     xs = [(torch.randn(n, channels + 6, generator=g) * 2).to(dtype) for n in lengths]  # the channels lie inside wider rows
     w = torch.randn(channels, taps, generator=g) * 0.7
     bias = torch.randn(channels, generator=g)
-    for unit_eps, b in ((None, bias), (1e-6, None)):
+    for unit_eps, b, moves in ((None, bias, False), (1e-6, None, False), (None, bias, True), (1e-6, None, True)):
         want = []
         for x in xs:
             y = PR.silu(PR.causal_conv(x[:, 3:3 + channels].double(), w.double(), None if b is None else b.double()))
@@ -77,14 +77,17 @@ def test_convolution_with_its_state_under_any_cutting(dtype, taps, channels, gro
         slots[:, :11] = 7.0  # what lies before the state is someone else's
         got = [[], []]
         cuts = [cuts_of(lengths[0], [1, 2, 3, 1, 5, 2, 9]), cuts_of(lengths[1], [2, 1, 1, 5])]
+        if moves:  # single tokens only: the convolution moves its state on itself
+            cuts = [cuts_of(n, [1]) for n in lengths]
         for i in range(max(len(c) for c in cuts)):
             live = [r for r in range(2) if i < len(cuts[r])]
             step = make_step([cuts[r][i] for r in live], [3 if r == 0 else 1 for r in live])
             rows = torch.cat([xs[r][cuts[r][i][0]:cuts[r][i][0] + cuts[r][i][1]] for r in live])
             out = torch.full((rows.shape[0], channels + 2), -5.0, dtype=torch.float32 if unit_eps else dtype, device=DEV)
             ops.causal_conv(dev(rows), 3, channels, dev(w), None if b is None else dev(b), slots, 11, step, out, 1,
-                            group=group, unit_eps=unit_eps, scaled_groups=2, group_scale=0.25)
-            ops.conv_state_update(dev(rows), 3, channels, taps, slots, 11, step)
+                            group=group, unit_eps=unit_eps, scaled_groups=2, group_scale=0.25, move_state=moves)
+            if not moves:
+                ops.conv_state_update(dev(rows), 3, channels, taps, slots, 11, step)
             assert float(out[:, 0].max()) == -5.0 and float(out[:, -1].max()) == -5.0
             at = 0
             for r in live:
@@ -92,7 +95,7 @@ def test_convolution_with_its_state_under_any_cutting(dtype, taps, channels, gro
                 got[r].append(out[at:at + n, 1:1 + channels].float().cpu())
                 at += n
         for r in range(2):
-            close(torch.cat(got[r]), want[r], dtype, f"request {r} unit={unit_eps}", bf16=1e-2)
+            close(torch.cat(got[r]), want[r], dtype, f"request {r} unit={unit_eps} moves={moves}", bf16=1e-2)
         assert float(slots[:, :11].min()) == 7.0
         if taps > 1:  # the other slots are untouched; the state holds the last inputs, oldest first
             assert float(slots[[0, 2, 4], 11:].abs().max()) == 0.0
@@ -207,8 +210,10 @@ def test_rotation_in_halves_norm_and_keys_written_as_values(dtype, nq, nkv, hd, 
     T = len(positions)
     cols = (nq + nkv) * hd + 5
     proj = (torch.randn(T, cols, generator=g) * 3).to(dtype)
-    q_in = proj[:, 2:2 + nq * hd].double().view(T, nq, hd)
-    k_in = proj[:, 2 + nq * hd:2 + (nq + nkv) * hd].double().view(T, nkv, hd)
+    bias = torch.randn(cols, generator=g) if mode == ops.NORM_AFTER_ROTATION else None
+    raw = proj if bias is None else (proj.double() + bias.double()).to(dtype)  # a projection with its bias, as stored
+    q_in = raw[:, 2:2 + nq * hd].double().view(T, nq, hd)
+    k_in = raw[:, 2 + nq * hd:2 + (nq + nkv) * hd].double().view(T, nkv, hd)
     pos = torch.tensor(positions)
     weighted = mode == ops.NORM_BEFORE_ROTATION
     qw, kw = torch.randn(hd, generator=g), torch.randn(hd, generator=g)
@@ -235,14 +240,15 @@ def test_rotation_in_halves_norm_and_keys_written_as_values(dtype, nq, nkv, hd, 
     q_out = torch.empty(T, nq * hd, dtype=dtype, device=DEV)
     ops.rotate_norm_write(dev(proj), 2, 2 + nq * hd, None, q_out, dev(qw) if weighted else None,
                           dev(kw) if weighted else None, 1e-5, 0.0, mode, rope, rot, dev(pos.int()),
-                          dev(torch.zeros(T, dtype=torch.int32)), dev(table), k_pages, v_pages, nq, nkv, hd)
+                          dev(torch.zeros(T, dtype=torch.int32)), dev(table), k_pages, v_pages, nq, nkv, hd,
+                          bias=None if bias is None else dev(bias))
     close(q_out.view(T, nq, hd), plain(q_in, qw), dtype, "queries")
     want_k = plain(k_in, kw)
     for t, p in enumerate(positions):
         page, slot = int(table[0, p // page_size]), p % page_size
         close(k_pages[page, :, slot], want_k[t], dtype, f"key at {p}")
         got_v = v_pages[page, :, slot // 16, :, slot % 16]
-        assert torch.equal(got_v.cpu(), proj[t, 2 + nq * hd:2 + (nq + nkv) * hd].view(nkv, hd)), f"value at {p}"
+        assert torch.equal(got_v.cpu(), raw[t, 2 + nq * hd:2 + (nq + nkv) * hd].view(nkv, hd)), f"value at {p}"
     untouched = [p for p in range(num_pages) if p not in {int(table[0, page]) for page in pages}]
     assert float(k_pages[untouched].abs().max()) == 0.0
 
@@ -267,6 +273,15 @@ def test_sandwich_on_a_32_bit_stream_with_a_scale_a_channel(dtype, width):
     parts = torch.randn(3, rows, width, generator=g)
     assert ops.add_rmsnorm_scaled(ops.SlicedSums(dev(parts), dtype), dev(w_post), 1e-5, 0.0, None, x) is None
     close(x, x0.double() + PR.rms_norm(parts.double().sum(0), 1e-5, w_post.double()), torch.float32, "partial sums")
+    # two branches with their weights, one stored and one as partial sums, normed as their sum
+    x = dev(x0.clone())
+    both = ops.BranchSum(dev(branch), ops.SlicedSums(dev(parts), dtype), -0.8, 1.3)
+    nxt = ops.add_rmsnorm_scaled(both, dev(w_post), 1e-5, 0.0, dev(scale), x, dev(w_next), 1e-5, 0.0)
+    mixed = -0.8 * branch.double() + 1.3 * parts.double().sum(0)
+    ref = x0.double() + PR.rms_norm(mixed, 1e-5, w_post.double()) * scale.double()
+    close(x, ref, torch.float32, "two branches")
+    close(nxt, PR.rms_norm(ref, 1e-5, w_next.double()), dtype, "the next norm after two branches")
+    close(ops.as_tensor(both), mixed, dtype, "two branches added up")
     # the norm that reads the stream and writes activations, whole and by rows
     close(ops.rmsnorm_cast(dev(x0), dev(w_next), 1e-5, 0.0, dtype), PR.rms_norm(x0.double(), 1e-5, w_next.double()), dtype)
     pick = torch.tensor([5, 0, 2], dtype=torch.int32)
