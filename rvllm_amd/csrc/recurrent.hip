@@ -415,6 +415,10 @@ extern "C" int rv_delta_rule(hipStream_t stream, const float* qkv, long long ld,
 // Selective scan.  LANES neighbouring lanes own a channel: lane `sub` holds the states sub * PER .. + PER.  A wave
 // holds 64 / LANES channels of one request and walks its tokens of this step in order, CHUNK at a time through
 // registers and LDS as the delta rule above; the step sizes and the gates' silu are worked out once a token there.
+// A channel's y is the sum of its states' products S C added as a balanced tree over the states in their order
+// (inside a lane first, then between the lanes), so that it has the same bits however the states are dealt to
+// lanes: a lane a state for prompts (a wave for every SIMD from one request), four states a lane for decoded
+// tokens (a channel's states then lie in one 16-byte read, and a wave covers four times the channels).
 //   x    T [tokens, ld_x]    the convolved, activated input      z   T [tokens, ld_z]   the gate's input
 //   dt   T [tokens, ld_dt]   the step's projection; step = softplus(dt + dt_bias[c])
 //   bc   T [tokens, ld_bc]   B at b_col, C at c_col, `n_state` each
@@ -430,6 +434,9 @@ selective_scan_kernel(const T* __restrict__ x, long long ld_x, const T* __restri
                       const float* __restrict__ A_log, const float* __restrict__ D, float* __restrict__ state,
                       long long slot_stride, long long s_off, const int* __restrict__ q_start,
                       const int* __restrict__ state_slot, T* __restrict__ out, int channels, int n_state) {
+  // Products and sums stay the separate operations they are written as (fmaf where one rounding is meant): a
+  // channel's tree of sums must have the same bits whether its products lie in one lane or in several.
+#pragma clang fp contract(off)
   constexpr int CPW = RV_WAVE / LANES;  // channels a wave
   constexpr int NP = PER * LANES;       // the states, padded
   constexpr int NB = (CHUNK * NP + RV_WAVE - 1) / RV_WAVE;
@@ -447,10 +454,17 @@ selective_scan_kernel(const T* __restrict__ x, long long ld_x, const T* __restri
   const int c = live ? ch : channels - 1;
   float* S_mem = state + (long long)state_slot[req] * slot_stride + s_off + (long long)c * n_state + sub * PER;
   float S[PER], A[PER];
+  const bool vec = PER == 4 && n_state % 4 == 0 && (((uintptr_t)S_mem & 15) == 0);
+  if (vec && sub * PER < n_state) {
+    const float4 v4 = *(const float4*)S_mem;
+    S[0] = v4.x, S[1 % PER] = v4.y, S[2 % PER] = v4.z, S[3 % PER] = v4.w;
+  } else {
+#pragma unroll
+    for (int e = 0; e < PER; ++e) S[e] = sub * PER + e < n_state ? S_mem[e] : 0.f;
+  }
 #pragma unroll
   for (int e = 0; e < PER; ++e) {
     const int n = sub * PER + e;
-    S[e] = n < n_state ? S_mem[e] : 0.f;
     A[e] = n < n_state ? -expf(A_log[(long long)c * n_state + n]) : 0.f;
   }
   const float skip = D[c];
@@ -505,31 +519,44 @@ selective_scan_kernel(const T* __restrict__ x, long long ld_x, const T* __restri
       const float step = sstep[t][cl];
       const float xv = sx[t][cl];
       const float sx_ = step * xv;
-      float y = 0.f;
+      float prod[PER];
 #pragma unroll
       for (int e = 0; e < PER; ++e) {
         S[e] = fmaf(rec_decay_exp<T>(step * A[e]), S[e], sx_ * sB[t][sub * PER + e]);
-        y = fmaf(S[e], sC[t][sub * PER + e], y);
+        prod[e] = S[e] * sC[t][sub * PER + e];  // a product of its own (no contraction here): see the pragma above
       }
-      y = rec_group_sum<LANES>(y);
+#pragma unroll
+      for (int w = 1; w < PER; w *= 2)
+#pragma unroll
+        for (int e = 0; e + w < PER; e += 2 * w) prod[e] += prod[e + w];
+      float y = rec_group_sum<LANES>(prod[0]);
       y = fmaf(skip, xv, y);
       if (live && sub == 0) out[(long long)(tb + t) * channels + ch] = rv_from_float<T>(y * sg[t][cl]);
     }
   }
   if (live) {
+    if (vec && sub * PER < n_state) {
+      *(float4*)S_mem = make_float4(S[0], S[1 % PER], S[2 % PER], S[3 % PER]);
+    } else {
 #pragma unroll
-    for (int e = 0; e < PER; ++e)
-      if (sub * PER + e < n_state) S_mem[e] = S[e];
+      for (int e = 0; e < PER; ++e)
+        if (sub * PER + e < n_state) S_mem[e] = S[e];
+    }
   }
 }
 
 #define REC_SCAN_PER_MAX 4
 
-// Lanes that share a channel: one a state up to 64 (every state costs an exponential a token, and a prompt of one
-// request wants a wave for every SIMD), then up to REC_SCAN_PER_MAX states a lane.
-extern "C" int rv_selective_scan_lanes(int n_state) {
+// Lanes that share a channel.  Prompts (`few` 0): one a state up to 64 (every state costs an exponential a token, and
+// a prompt of one request wants a wave for every SIMD), then up to REC_SCAN_PER_MAX states a lane.  Steps of decoded
+// tokens (`few` 1): REC_SCAN_PER_MAX states a lane.
+extern "C" int rv_selective_scan_lanes(int n_state, int few) {
   int lanes = 1;
-  while (lanes < RV_WAVE && lanes < n_state) lanes *= 2;
+  if (few) {
+    while (lanes < RV_WAVE && rv_div_up(n_state, lanes) > REC_SCAN_PER_MAX) lanes *= 2;
+  } else {
+    while (lanes < RV_WAVE && lanes < n_state) lanes *= 2;
+  }
   return lanes;
 }
 
@@ -542,39 +569,41 @@ extern "C" int rv_selective_scan(hipStream_t stream, const void* x, long long ld
   RV_CHECK(x && z && dt && dt_bias && bc && A_log && D && state && q_start && state_slot && out,
            "selective_scan: null argument");
   RV_CHECK(channels > 0 && n_state > 0 && num_requests >= 0, "selective_scan: bad sizes");
-  const int lanes = rv_selective_scan_lanes(n_state);
+  const bool few = longest <= 2;
+  const int lanes = rv_selective_scan_lanes(n_state, few);
   const int per = rv_div_up(n_state, lanes);
   RV_CHECK(per <= REC_SCAN_PER_MAX, "selective_scan: %d states a channel are more than %d", n_state,
            REC_SCAN_PER_MAX * RV_WAVE);
   if (num_requests == 0) return 0;
   dim3 grid(rv_div_up(channels, RV_WAVE / lanes), num_requests), block(RV_WAVE);
-  const bool few = longest <= 2;
 #define RV_SS(T, PER, LANES, CHUNK)                                                                                \
   selective_scan_kernel<T, PER, LANES, CHUNK><<<grid, block, 0, stream>>>(                                         \
       (const T*)x, ld_x, (const T*)z, ld_z, (const T*)dt, ld_dt, dt_bias, (const T*)bc, ld_bc, b_col, c_col, A_log, \
       D, state, slot_stride, s_off, q_start, state_slot, (T*)out, channels, n_state)
-#define RV_SS_L(T, PER, LANES, CHUNK)     \
-  do {                                    \
-    if (few) RV_SS(T, PER, LANES, 2);     \
-    else RV_SS(T, PER, LANES, CHUNK);     \
-  } while (0)
-#define RV_SS_T(T)                                    \
-  do {                                                \
-    if (lanes == 1) RV_SS_L(T, 1, 1, 16);             \
-    else if (lanes == 2) RV_SS_L(T, 1, 2, 16);        \
-    else if (lanes == 4) RV_SS_L(T, 1, 4, 16);        \
-    else if (lanes == 8) RV_SS_L(T, 1, 8, 16);        \
-    else if (lanes == 16) RV_SS_L(T, 1, 16, 16);      \
-    else if (lanes == 32) RV_SS_L(T, 1, 32, 16);      \
-    else if (per <= 1) RV_SS_L(T, 1, 64, 16);         \
-    else if (per <= 2) RV_SS_L(T, 2, 64, 8);          \
-    else RV_SS_L(T, 4, 64, 4);                        \
+#define RV_SS_T(T)                                     \
+  do {                                                 \
+    if (few) {                                         \
+      if (lanes == 1) RV_SS(T, 4, 1, 2);               \
+      else if (lanes == 2) RV_SS(T, 4, 2, 2);          \
+      else if (lanes == 4) RV_SS(T, 4, 4, 2);          \
+      else if (lanes == 8) RV_SS(T, 4, 8, 2);          \
+      else if (lanes == 16) RV_SS(T, 4, 16, 2);        \
+      else if (lanes == 32) RV_SS(T, 4, 32, 2);        \
+      else RV_SS(T, 4, 64, 2);                         \
+    } else if (lanes == 1) RV_SS(T, 1, 1, 16);         \
+    else if (lanes == 2) RV_SS(T, 1, 2, 16);           \
+    else if (lanes == 4) RV_SS(T, 1, 4, 16);           \
+    else if (lanes == 8) RV_SS(T, 1, 8, 16);           \
+    else if (lanes == 16) RV_SS(T, 1, 16, 16);         \
+    else if (lanes == 32) RV_SS(T, 1, 32, 16);         \
+    else if (per <= 1) RV_SS(T, 1, 64, 16);            \
+    else if (per <= 2) RV_SS(T, 2, 64, 8);             \
+    else RV_SS(T, 4, 64, 4);                           \
   } while (0)
   if (dtype == RV_F32) RV_SS_T(float);
   else if (dtype == RV_BF16) RV_SS_T(bf16_t);
   else return rv_fail("selective_scan: unsupported dtype %d", dtype);
 #undef RV_SS_T
-#undef RV_SS_L
 #undef RV_SS
   RV_LAUNCH_CHECK("selective_scan");
   return 0;

@@ -55,26 +55,29 @@ def cuts_of(total, sizes):
 # --------------------------------------------------------------------------
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("taps,channels,group", [(4, 96, 32), (1, 40, 40), (2, 70, 7), (5, 300, 100), (3, 64, 64)])
-def test_convolution_with_its_state_under_any_cutting(dtype, taps, channels, group):
+@pytest.mark.parametrize("aligned", [False, True])
+def test_convolution_with_its_state_under_any_cutting(dtype, taps, channels, group, aligned):
     """Two requests in two slots out of five; portions of 1, 2, 3 and more tokens, shorter than the taps too; the
-    state row that a portion leaves is what the next one starts from; with and without unit length and bias."""
+    state row that a portion leaves is what the next one starts from; with and without unit length and bias.
+    ``aligned``: channels, rows and state on 16-byte boundaries, or at odd places."""
     g = torch.Generator().manual_seed(taps * 1000 + channels)
     lengths = [23, 9]
-    xs = [(torch.randn(n, channels + 6, generator=g) * 2).to(dtype) for n in lengths]  # the channels lie inside wider rows
+    c_in, c_out, s_off, pad = (8, 8, 16, 16) if aligned else (3, 1, 11, 6)
+    xs = [(torch.randn(n, channels + pad, generator=g) * 2).to(dtype) for n in lengths]  # the channels lie inside wider rows
     w = torch.randn(channels, taps, generator=g) * 0.7
     bias = torch.randn(channels, generator=g)
     for unit_eps, b, moves in ((None, bias, False), (1e-6, None, False), (None, bias, True), (1e-6, None, True)):
         want = []
         for x in xs:
-            y = PR.silu(PR.causal_conv(x[:, 3:3 + channels].double(), w.double(), None if b is None else b.double()))
+            y = PR.silu(PR.causal_conv(x[:, c_in:c_in + channels].double(), w.double(), None if b is None else b.double()))
             y = y.to(dtype).double()  # the activated output is rounded to the activations' type once
             if unit_eps is not None:
                 y = PR.unit(y.view(-1, channels // group, group), unit_eps)
                 y[:, :2] *= 0.25
                 y = y.reshape(-1, channels)
             want.append(y)
-        slots = torch.zeros(5, 11 + (taps - 1) * channels, device=DEV)
-        slots[:, :11] = 7.0  # what lies before the state is someone else's
+        slots = torch.zeros(5, s_off + (taps - 1) * channels, device=DEV)
+        slots[:, :s_off] = 7.0  # what lies before the state is someone else's
         got = [[], []]
         cuts = [cuts_of(lengths[0], [1, 2, 3, 1, 5, 2, 9]), cuts_of(lengths[1], [2, 1, 1, 5])]
         if moves:  # single tokens only: the convolution moves its state on itself
@@ -83,23 +86,25 @@ def test_convolution_with_its_state_under_any_cutting(dtype, taps, channels, gro
             live = [r for r in range(2) if i < len(cuts[r])]
             step = make_step([cuts[r][i] for r in live], [3 if r == 0 else 1 for r in live])
             rows = torch.cat([xs[r][cuts[r][i][0]:cuts[r][i][0] + cuts[r][i][1]] for r in live])
-            out = torch.full((rows.shape[0], channels + 2), -5.0, dtype=torch.float32 if unit_eps else dtype, device=DEV)
-            ops.causal_conv(dev(rows), 3, channels, dev(w), None if b is None else dev(b), slots, 11, step, out, 1,
-                            group=group, unit_eps=unit_eps, scaled_groups=2, group_scale=0.25, move_state=moves)
+            out = torch.full((rows.shape[0], channels + 2 * c_out), -5.0, dtype=torch.float32 if unit_eps else dtype,
+                             device=DEV)
+            ops.causal_conv(dev(rows), c_in, channels, dev(w), None if b is None else dev(b), slots, s_off, step, out,
+                            c_out, group=group, unit_eps=unit_eps, scaled_groups=2, group_scale=0.25, move_state=moves)
             if not moves:
-                ops.conv_state_update(dev(rows), 3, channels, taps, slots, 11, step)
-            assert float(out[:, 0].max()) == -5.0 and float(out[:, -1].max()) == -5.0
+                ops.conv_state_update(dev(rows), c_in, channels, taps, slots, s_off, step)
+            assert float(out[:, :c_out].max()) == -5.0 and float(out[:, -c_out:].max()) == -5.0
             at = 0
             for r in live:
                 n = cuts[r][i][1]
-                got[r].append(out[at:at + n, 1:1 + channels].float().cpu())
+                got[r].append(out[at:at + n, c_out:c_out + channels].float().cpu())
                 at += n
         for r in range(2):
             close(torch.cat(got[r]), want[r], dtype, f"request {r} unit={unit_eps} moves={moves}", bf16=1e-2)
-        assert float(slots[:, :11].min()) == 7.0
+        assert float(slots[:, :s_off].min()) == 7.0
         if taps > 1:  # the other slots are untouched; the state holds the last inputs, oldest first
-            assert float(slots[[0, 2, 4], 11:].abs().max()) == 0.0
-            close(slots[3, 11:].view(taps - 1, channels), xs[0][-(taps - 1):, 3:3 + channels].float(), torch.float32)
+            assert float(slots[[0, 2, 4], s_off:].abs().max()) == 0.0
+            close(slots[3, s_off:].view(taps - 1, channels), xs[0][-(taps - 1):, c_in:c_in + channels].float(),
+                  torch.float32)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -146,7 +151,7 @@ def test_delta_rule_whole_and_cut_give_the_same_bits(dtype, heads, kv_heads, dk,
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("channels,n_state", [(48, 6), (100, 33), (7, 1), (320, 16), (65, 200)])
+@pytest.mark.parametrize("channels,n_state", [(48, 6), (100, 33), (7, 1), (328, 16), (65, 200)])
 def test_selective_scan_whole_and_cut_and_two_requests(dtype, channels, n_state):
     g = torch.Generator().manual_seed(channels + n_state)
     T = [29, 6]
@@ -202,7 +207,7 @@ def test_output_norm_a_head_with_a_shared_weight_and_a_silu_gate(dtype, heads, d
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("nq,nkv,hd,rot,page_size", [(4, 2, 32, 16, 16), (3, 3, 20, 20, 32), (5, 1, 12, 6, 16),
-                                                     (2, 1, 96, 96, 64), (2, 2, 272, 0, 16), (1, 1, 512, 130, 16)])
+                                                     (2, 1, 80, 80, 64), (2, 2, 272, 0, 16), (1, 1, 512, 130, 16)])
 @pytest.mark.parametrize("mode", [ops.NORM_AFTER_ROTATION, ops.NORM_BEFORE_ROTATION, ops.NORM_NONE])
 def test_rotation_in_halves_norm_and_keys_written_as_values(dtype, nq, nkv, hd, rot, page_size, mode):
     g = torch.Generator().manual_seed(hd + rot)
